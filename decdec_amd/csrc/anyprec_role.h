@@ -1,0 +1,214 @@
+// Any-precision bitplane GEMV role (batch 1):  out[n] += sum_c lut[n][idx(n, c)] * x[c].
+//
+// Weight layout (reference decdec_extension/anyprec.cu:297-329 and :411-475): qweight[p][n][w],
+// plane 0 = MSB of the LUT index, w = 32*i + t for 1024-channel chunk i and word t; bit
+// 31 - (8j + e) of word (i, t) belongs to channel 1024 i + 8 eff j + 8 t + e, j in [0,4), e in [0,8),
+// eff = 32 for full chunks and (K % 1024)/32 for a tail chunk.
+//
+// Mapping: a wave owns one slice of 64 consecutive words (2048 channels) of the row and keeps the
+// matching 32 activations per lane in registers for every row it visits; the S slices of a row sit in
+// S waves of the same workgroup and are summed in LDS, so each output receives exactly one atomic add
+// (the reference's accumulate-into-output contract).  Weights stream from HBM as coalesced 256-byte
+// wave loads per plane; several rows are in flight per wave.
+//
+// The 3-bit path keeps the row's 8-entry LUT in four VGPRs as two byte tables and looks weights up
+// with v_perm_b32 (four table lookups per instruction), then multiplies with v_dot2_f32_f16 /
+// v_dot2_f32_bf16 into an fp32 accumulator: no LDS traffic in the inner loop.  Other bit widths use
+// a per-wave LDS copy of the row's LUT.
+#pragma once
+#include "common.h"
+
+namespace decdec {
+
+struct AnyprecParams {
+    const void* x;
+    const uint32_t* qweight;
+    const void* lut;
+    void* out;
+    uint32_t N, K, W;      // W = K / 32 words per row per plane
+    uint32_t S;            // slices (waves) per row handled inside one workgroup (<= 16)
+    uint32_t sgroups;      // slice groups (> 1 only when ceil(W/64) > 16, i.e. K > 32768)
+    uint32_t rg;           // row groups per workgroup
+    uint32_t rpw;          // rows per wave (even)
+    uint32_t x_aligned;    // activation pointer is 16-byte aligned
+};
+
+__host__ __device__ inline size_t anyprec_lds_bytes(uint32_t S, uint32_t rg, uint32_t rpw, int bits) {
+    size_t b = (size_t)S * rg * rpw * 4;
+    if (bits != 3) b += (size_t)S * rg * 256 * 4;     // per-wave LUT copy
+    return b;
+}
+
+template <int DT>
+__device__ __forceinline__ float dot2_acc(uint32_t w, uint32_t x, float acc) {
+    if constexpr (DT == kFP16) {
+        return __builtin_amdgcn_fdot2(*(half2_t*)&w, *(half2_t*)&x, acc, false);
+    } else {
+        return __builtin_amdgcn_fdot2_f32_bf16(*(bf16x2_t*)&w, *(bf16x2_t*)&x, acc, false);
+    }
+}
+
+// Load the 32 activations that belong to word `wi` of a row, arranged for the decoders below:
+// xp[e][0] = (x[j=3][e], x[j=2][e]),  xp[e][1] = (x[j=1][e], x[j=0][e])  as packed 16-bit pairs.
+__device__ __forceinline__ void anyprec_load_x(const AnyprecParams& p, uint32_t wi, uint32_t (&xp)[8][2]) {
+    const uint32_t i = wi >> 5, t = wi & 31u;
+    const uint32_t eff = (i == p.K / 1024u) ? (p.K % 1024u) / 32u : 32u;
+    uint32_t xr[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const size_t c0 = (size_t)1024 * i + (size_t)8 * eff * j + (size_t)8 * t;
+        const uint16_t* src = (const uint16_t*)p.x + c0;
+        if (p.x_aligned) {
+            const u32x4 v = *(const u32x4*)src;
+            xr[j][0] = v[0]; xr[j][1] = v[1]; xr[j][2] = v[2]; xr[j][3] = v[3];
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xr[j][q] = (uint32_t)src[2 * q] | ((uint32_t)src[2 * q + 1] << 16);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+        xp[e][0] = __builtin_amdgcn_perm(xr[2][e >> 1], xr[3][e >> 1], sel);   // lo = j3, hi = j2
+        xp[e][1] = __builtin_amdgcn_perm(xr[0][e >> 1], xr[1][e >> 1], sel);   // lo = j1, hi = j0
+    }
+}
+
+// One word of a 3-bit row: 32 weights looked up through byte-permutes and dotted with xp.
+// lut4 holds the row's eight 16-bit LUT entries (two per dword).
+template <int DT>
+__device__ __forceinline__ float anyprec3_word(uint32_t q0, uint32_t q1, uint32_t q2, const u32x4 lut4,
+                                               const uint32_t (&xp)[8][2], float acc) {
+    // byte tables: LO = low bytes of entries 0..7, HI = high bytes
+    const uint32_t lo0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x06040200u);
+    const uint32_t hi0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x07050301u);
+    const uint32_t lo1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x06040200u);
+    const uint32_t hi1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x07050301u);
+    // index words: nibble n of T_o carries the 3-bit index of bit 4n+o (o = 3..0), either at nibble
+    // bits 3..1 (T3, T1) or 2..0 (T2, T0); the unused nibble bit is garbage and masked below.
+    const uint32_t r1 = q1 >> 1, r2 = q2 >> 2, l0 = q0 << 2, l1 = q1 << 1;
+    const uint32_t m8 = 0x88888888u, m4 = 0x44444444u, m2 = 0x22222222u;
+    const uint32_t t3 = (q0 & m8) | (r1 & m4) | (r2 & ~(m8 | m4));
+    const uint32_t t2 = (q0 & m4) | (r1 & m2) | (r2 & ~(m4 | m2));
+    const uint32_t t1 = (l0 & m8) | (l1 & m4) | (q2 & ~(m8 | m4));
+    const uint32_t t0 = (l0 & m4) | (l1 & m2) | (q2 & ~(m4 | m2));
+    const uint32_t k7 = 0x07070707u;
+    // selector bytes 0..3 <-> j = 3..0; element e per selector as listed
+    const uint32_t sel[8] = {
+        (t3 >> 5) & k7,   // e = 0
+        (t2 >> 4) & k7,   // e = 1
+        (t1 >> 5) & k7,   // e = 2
+        (t0 >> 4) & k7,   // e = 3
+        (t3 >> 1) & k7,   // e = 4
+        t2 & k7,          // e = 5
+        (t1 >> 1) & k7,   // e = 6
+        t0 & k7,          // e = 7
+    };
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t L = __builtin_amdgcn_perm(lo1, lo0, sel[e]);
+        const uint32_t H = __builtin_amdgcn_perm(hi1, hi0, sel[e]);
+        const uint32_t w32 = __builtin_amdgcn_perm(H, L, 0x05010400u);   // weights j3, j2
+        const uint32_t w10 = __builtin_amdgcn_perm(H, L, 0x07030602u);   // weights j1, j0
+        acc = dot2_acc<DT>(w32, xp[e][0], acc);
+        acc = dot2_acc<DT>(w10, xp[e][1], acc);
+    }
+    return acc;
+}
+
+// Generic bit width: indices assembled bytewise, weights from a per-wave LDS copy of the LUT (fp32).
+template <int DT, int BITS>
+__device__ __forceinline__ float anyprec_generic_word(const uint32_t (&q)[BITS], const float* wlut,
+                                                      const uint32_t (&xp)[8][2], float acc) {
+#pragma unroll
+    for (int o = 0; o < 8; ++o) {
+        uint32_t u = 0;
+#pragma unroll
+        for (int pl = 0; pl < BITS; ++pl) u |= ((q[pl] >> o) & 0x01010101u) << (BITS - 1 - pl);
+        const int e = 7 - o;                               // byte k of u <-> j = 3 - k
+        const float w3 = wlut[u & 0xFFu], w2 = wlut[(u >> 8) & 0xFFu];
+        const float w1 = wlut[(u >> 16) & 0xFFu], w0 = wlut[u >> 24];
+        float x3, x2, x1, x0;
+        if constexpr (DT == kFP16) {
+            const half2_t a = *(const half2_t*)&xp[e][0], b = *(const half2_t*)&xp[e][1];
+            x3 = (float)a[0]; x2 = (float)a[1]; x1 = (float)b[0]; x0 = (float)b[1];
+        } else {
+            x3 = __uint_as_float(xp[e][0] << 16); x2 = __uint_as_float(xp[e][0] & 0xFFFF0000u);
+            x1 = __uint_as_float(xp[e][1] << 16); x0 = __uint_as_float(xp[e][1] & 0xFFFF0000u);
+        }
+        acc += w3 * x3; acc += w2 * x2; acc += w1 * x1; acc += w0 * x0;
+    }
+    return acc;
+}
+
+template <int DT, int BITS>
+__device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
+    using E = Elem<DT>;
+    constexpr int RB = 4;                                   // rows per load batch
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t s = wave % p.S, g = wave / p.S;
+    const uint32_t rows_per_block = p.rg * p.rpw;
+    const uint32_t sgrp = bid % p.sgroups, tile = bid / p.sgroups;
+    const uint32_t block_row0 = tile * rows_per_block;
+    const bool wave_active = g < p.rg;
+    const uint32_t wi = (sgrp * p.S + s) * kWave + lane;    // word index inside the row
+    const bool lane_ok = wave_active && (wi < p.W);
+    float* part = (float*)smem;                             // [rows_per_block][S]
+    float* wlut = part + (size_t)rows_per_block * p.S + (size_t)wave * 256;
+
+    uint32_t xp[8][2];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { xp[e][0] = 0u; xp[e][1] = 0u; }
+    if (lane_ok) anyprec_load_x(p, wi, xp);
+
+    if (wave_active) {
+        const uint32_t row0 = block_row0 + g * p.rpw;
+        const size_t plane_stride = (size_t)p.N * p.W;
+        for (uint32_t rb = 0; rb < p.rpw; rb += RB) {
+            uint32_t q[RB][BITS];
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const uint32_t row = row0 + rb + r;
+                const bool ok = lane_ok && (rb + r < p.rpw) && (row < p.N);
+#pragma unroll
+                for (int pl = 0; pl < BITS; ++pl)
+                    q[r][pl] = ok ? p.qweight[pl * plane_stride + (size_t)row * p.W + wi] : 0u;
+            }
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const uint32_t row = row0 + rb + r;
+                if (rb + r >= p.rpw) break;                 // uniform
+                float acc = 0.f;
+                if (row < p.N) {                            // uniform
+                    if constexpr (BITS == 3) {
+                        const u32x4 lut4 = *(const u32x4*)((const uint16_t*)p.lut + (size_t)row * 8);
+                        acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lut4, xp, 0.f);
+                    } else {
+                        constexpr int L = 1 << BITS;
+                        __builtin_amdgcn_wave_barrier();
+                        for (int v = lane; v < L; v += kWave) wlut[v] = E::load(p.lut, (size_t)row * L + v);
+                        __builtin_amdgcn_wave_barrier();
+                        acc = anyprec_generic_word<DT, BITS>(q[r], wlut, xp, 0.f);
+                    }
+                }
+                acc = wave_sum(acc);
+                if (lane == 0) part[(size_t)(g * p.rpw + rb + r) * p.S + s] = acc;
+            }
+        }
+    }
+    __syncthreads();
+    // one atomic per output pair
+    for (uint32_t t = tid; t < rows_per_block / 2; t += blockDim.x) {
+        const uint32_t r = 2 * t, row = block_row0 + r;
+        if (row >= p.N) continue;
+        float v0 = 0.f, v1 = 0.f;
+        for (uint32_t ss = 0; ss < p.S; ++ss) {
+            v0 += part[(size_t)r * p.S + ss];
+            v1 += part[(size_t)(r + 1) * p.S + ss];
+        }
+        if (row + 1 < p.N) E::atomic_add2(p.out, row, v0, v1);
+        else E::atomic_add1(p.out, row, v0);
+    }
+}
+
+}  // namespace decdec

@@ -1,0 +1,771 @@
+// C-ABI layer of libdecdec_hip.so: argument validation, DEC context / config objects, launch
+// planning, and the two ways of running DEC next to a base GEMV (one fused launch, or the
+// reference's two-stream fork/join).  Declarations and reference citations: include/decdec_hip.h.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_set>
+
+#include "../../include/decdec_hip.h"
+#include "launch.h"
+
+using namespace decdec;
+
+namespace {
+
+enum { kOk = 0, kInvalid = 1, kHipError = 2, kUnsupported = 3 };
+
+thread_local std::string g_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
+#define DD_HIP(expr)                                                                         \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess) return fail(kHipError, "HIP error in %s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+#define DD_CHECK(cond, ...)                          \
+    do {                                             \
+        if (!(cond)) return fail(kInvalid, __VA_ARGS__); \
+    } while (0)
+
+// ---- options -------------------------------------------------------------------------------------
+struct Options {
+    int fusion = 1;
+    int host_noncoherent = 0;
+    int anyprec_rpw = 0;
+    int lutgemm_npb = 0;
+    int sqllm_ktiles = 0;
+    int dec_lds_reduce = 1;
+} g_opt;
+
+int* option_slot(const char* name) {
+    if (!name) return nullptr;
+    if (!strcmp(name, "fusion")) return &g_opt.fusion;
+    if (!strcmp(name, "host_noncoherent")) return &g_opt.host_noncoherent;
+    if (!strcmp(name, "anyprec_rpw")) return &g_opt.anyprec_rpw;
+    if (!strcmp(name, "lutgemm_npb")) return &g_opt.lutgemm_npb;
+    if (!strcmp(name, "sqllm_ktiles")) return &g_opt.sqllm_ktiles;
+    if (!strcmp(name, "dec_lds_reduce")) return &g_opt.dec_lds_reduce;
+    return nullptr;
+}
+
+// ---- soft-float conversions for the host-side threshold arithmetic ---------------------------------
+float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+float h2f(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 0x3FFu;
+    if (e == 0) { const float v = (float)m * 5.9604644775390625e-08f; return sign ? -v : v; }
+    if (e == 31) return bits_f32(sign | 0x7F800000u | (m << 13));
+    return bits_f32(sign | ((e + 112u) << 23) | (m << 13));
+}
+uint16_t f2h(float f) {   // round to nearest, ties to even
+    const uint32_t u = f32_bits(f), sign = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);
+    if (a >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u);
+    if (a <= 0x33000000u) return (uint16_t)sign;
+    const int e = (int)(a >> 23) - 127;
+    uint32_t m = (a & 0x7FFFFFu) | 0x800000u, base = 0;
+    int shift = 13;
+    if (e < -14) shift += -14 - e; else { base = (uint32_t)(e + 15) << 10; m &= 0x7FFFFFu; }
+    uint32_t q = m >> shift;
+    const uint32_t rem = m & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) ++q;
+    return (uint16_t)(sign | (base + q));
+}
+float b2f(uint16_t b) { return bits_f32((uint32_t)b << 16); }
+uint16_t f2b(float f) {
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+float round_to(float v, int dt) {
+    if (dt == DECDEC_FP16) return h2f(f2h(v));
+    if (dt == DECDEC_BF16) return b2f(f2b(v));
+    return v;
+}
+float load_host(const void* p, int dt, size_t i) {
+    if (dt == DECDEC_FP16) return h2f(((const uint16_t*)p)[i]);
+    if (dt == DECDEC_BF16) return b2f(((const uint16_t*)p)[i]);
+    return ((const float*)p)[i];
+}
+size_t dtype_size(int dt) { return dt == DECDEC_FP32 ? 4 : 2; }
+bool dtype_ok(int dt) { return dt == DECDEC_FP32 || dt == DECDEC_FP16 || dt == DECDEC_BF16; }
+
+// The selector's 32 bucket floors (reference dec.cu:117-130): each step rounded exactly where the
+// reference's typed arithmetic rounds.  volatile keeps the compiler from contracting or reassociating.
+void bucket_floors(float a, float b, int dt, float* out) {
+    volatile float diff = round_to(b - a, dt);
+    for (int i = 0; i < kBuckets; ++i) {
+        if (i < kBuckets / 2) {
+            volatile float prod = diff * (float)i;
+            volatile float quo = prod / (float)(kBuckets / 2 - 1);
+            volatile float step = round_to(quo, dt);
+            out[i] = round_to(a + step, dt);
+        } else {
+            volatile float prod = b * (float)(kBuckets - i - 1);
+            volatile float quo = prod / (float)(kBuckets - kBuckets / 2);
+            out[i] = round_to(quo, dt);
+        }
+    }
+}
+
+// ---- reference launch geometry (dec_config.cu:34-115), reported by read_dec_config ------------------
+uint32_t cdiv(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+int reference_geometry(uint32_t K, uint32_t N, uint32_t n_tb, uint32_t k_chunk, int dt, uint32_t max_smem,
+                       decdec_config_info* o) {
+    const uint32_t total = N / 8;
+    uint32_t cpt = cdiv(cdiv(total, n_tb), 32) * 32, bx;
+    if (cpt > 256) {
+        const uint32_t times = cdiv(cpt, 256);
+        bx = cdiv(total / n_tb / times, 32) * 32;
+        cpt = bx * times;
+    } else {
+        bx = cpt;
+    }
+    if (bx == 0) return 1;
+    const uint32_t num_blocks = cdiv(total, cpt), by = 1024 / bx, num_chunks = cdiv(K, 1024);
+    const uint32_t item = (uint32_t)dtype_size(dt);
+    const uint32_t rows = k_chunk * num_chunks;
+    const uint32_t row_select = k_chunk * 32 * 4 + 1024 * item;
+    uint32_t dec_req = rows * 4 + 8 * bx * by * item + bx * 8 * item + rows * item;
+    uint32_t dyn = std::max(row_select, dec_req);
+    int status = 0;
+    if (dyn + 128 > max_smem) {
+        dec_req = 8 * bx * by * item + bx * 8 * item;
+        dyn = std::max(row_select, dec_req);
+        status = (dyn + 128 > max_smem) ? -1 : 1;
+    }
+    o->num_chunks = (int)num_chunks; o->chunk_size = 1024; o->k_chunk = (int)k_chunk;
+    o->channels_per_tb = (int)cpt; o->n_tb = (int)std::min(std::max(num_chunks, num_blocks), n_tb);
+    o->block_dim_x = (int)bx; o->block_dim_y = (int)by; o->shared_memory_size = (int)dyn;
+    o->reduced_shared_memory = status == 1;
+    return status == -1 ? 2 : 0;
+}
+
+// ---- objects ---------------------------------------------------------------------------------------
+struct Context {
+    int dt;
+    uint32_t num_tb;
+    uint64_t buffer_numel;
+    int32_t* rows;
+    void* acts;
+    hipStream_t sub_stream;
+    hipEvent_t event;
+};
+
+struct DecPlan {
+    uint32_t cg, sg, nseg, vec, segs_per_block, slots, lds_reduce;
+    size_t lds;
+};
+
+struct Config {
+    int dt;
+    Context* ctx;
+    const uint32_t* residual_dev;   // device-visible residual
+    void* residual_host;            // owned pinned allocation (nullptr when borrowed from the device)
+    void* scales_dev;               // owned device copy
+    const void* thresholds_host;    // borrowed
+    uint32_t K, N, M, k_chunk, max_smem;
+    decdec_config_info info;
+    DecPlan plan;
+    hipEvent_t e1, e2;
+};
+
+std::mutex g_mu;
+std::unordered_set<uint64_t> g_contexts, g_configs;
+
+Context* get_context(uint64_t h) {
+    std::lock_guard<std::mutex> l(g_mu);
+    return g_contexts.count(h) ? reinterpret_cast<Context*>(h) : nullptr;
+}
+Config* get_config(uint64_t h) {
+    std::lock_guard<std::mutex> l(g_mu);
+    return g_configs.count(h) ? reinterpret_cast<Config*>(h) : nullptr;
+}
+
+constexpr size_t kLdsBudget = 60 * 1024;
+
+// Split the DEC work of one layer over at most `budget` workgroups: cg chunk groups x sg segment
+// groups, minimising the largest per-workgroup share; ties prefer fewer chunk groups (= fewer atomic
+// adds per output).  The row list of a workgroup must fit in LDS.
+int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, bool aligned16, DecPlan* pl) {
+    const uint32_t num_chunks = cdiv(K, 1024);
+    uint32_t vec = 1;
+    if (aligned16 && M % 4 == 0 && M >= 256) vec = 4;
+    else if (aligned16 && M % 2 == 0 && M >= 128) vec = 2;
+    const uint32_t nseg = cdiv(M, 64 * vec);
+    budget = std::max(1u, budget);
+    uint64_t best_cost = ~0ull;
+    uint32_t best_cg = 0, best_sg = 0;
+    size_t best_lds = 0;
+    uint32_t best_red = 0;
+    for (uint32_t cg = 1; cg <= num_chunks; ++cg) {
+        const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
+        for (uint32_t sg = 1; sg <= sg_max; ++sg) {
+            const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
+            const uint32_t slots = cpb * std::max(k_chunk, 1u);
+            uint32_t red = g_opt.dec_lds_reduce ? 1u : 0u;
+            size_t lds = dec_lds_bytes(slots, spb, vec, red);
+            if (lds > kLdsBudget && red) { red = 0; lds = dec_lds_bytes(slots, spb, vec, 0); }
+            if (lds > kLdsBudget) continue;
+            // per-workgroup critical path: sequential chunk selections + (chunk, segment) fetch units;
+            // going over the workgroup budget is a last resort
+            uint64_t cost = (uint64_t)cpb * spb * 1000 + (uint64_t)cpb * 600 + (uint64_t)cg * 10 +
+                            (cg * sg > budget ? 500000ull : 0);
+            if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; best_red = red; }
+        }
+    }
+    if (best_cg == 0) return 1;
+    pl->cg = best_cg; pl->sg = best_sg; pl->nseg = nseg; pl->vec = vec;
+    pl->segs_per_block = cdiv(nseg, best_sg);
+    pl->slots = cdiv(num_chunks, best_cg) * std::max(k_chunk, 1u);
+    pl->lds_reduce = best_red; pl->lds = best_lds;
+    return 0;
+}
+
+int setup_config(Config* c, uint32_t k_chunk) {
+    Context* ctx = c->ctx;
+    c->k_chunk = k_chunk;
+    memset(&c->info, 0, sizeof(c->info));
+    const int st = reference_geometry(c->K, c->N, std::max(1u, ctx->num_tb), k_chunk, c->dt, c->max_smem, &c->info);
+    if (st == 1) return fail(kInvalid, "DECConfig: output size %u is too small for the DEC launch geometry", c->N);
+    const uint64_t k = (uint64_t)k_chunk * c->K / 1024;
+    // reference dec_config.cu:180-181
+    DD_CHECK(ctx->buffer_numel >= k, "DECContext buffer size is too small for the given k_chunk.");
+    DD_CHECK(k_chunk <= 1024, "k_chunk must not exceed the chunk size (1024), got %u", k_chunk);
+    const bool aligned16 = ((uintptr_t)c->residual_dev % 16) == 0;
+    if (plan_dec(c->K, c->M, k_chunk, std::max(1u, ctx->num_tb), aligned16, &c->plan))
+        return fail(kUnsupported, "DEC launch plan does not fit in LDS (k_chunk=%u, K=%u)", k_chunk, c->K);
+    c->info.hip_dec_blocks = (int)(c->plan.cg * c->plan.sg);
+    c->info.hip_chunk_groups = (int)c->plan.cg;
+    c->info.hip_segment_groups = (int)c->plan.sg;
+    c->info.hip_vec_words = (int)c->plan.vec;
+    c->info.hip_lds_bytes = (int)c->plan.lds;
+    c->info.hip_slots_per_block = (int)c->plan.slots;
+    c->info.hip_lds_reduce = (int)c->plan.lds_reduce;
+    c->info.hip_residual_on_host = c->residual_host != nullptr;
+    return kOk;
+}
+
+// Fill the kernel parameters of one DEC call.  Returns 1 when there is nothing to do (k == 0).
+int fill_dec_params(const Config* c, const void* input, void* output, bool fused_select, DecParams* p) {
+    const uint64_t k = (uint64_t)c->k_chunk * c->K / 1024;       // reference decdec.cu:50
+    if (k == 0) return 1;                                        // reference decdec.cu:52-54
+    memset(p, 0, sizeof(*p));
+    p->residual = c->residual_dev; p->scales = c->scales_dev; p->x = input;
+    p->sel_rows = c->ctx->rows; p->sel_acts = c->ctx->acts; p->out = output;
+    if (fused_select) {
+        // thresholds[0] and thresholds[k-1] are read on the host at call time (reference decdec.cu:66-67)
+        const float a = load_host(c->thresholds_host, c->dt, 0);
+        const float b = load_host(c->thresholds_host, c->dt, (size_t)k - 1);
+        bucket_floors(a, b, c->dt, p->floors);
+    }
+    p->K = c->K; p->N = c->N; p->M = c->M;
+    p->num_chunks = cdiv(c->K, 1024); p->k_chunk = c->k_chunk; p->k_total = (uint32_t)k;
+    p->cg = c->plan.cg; p->sg = c->plan.sg; p->nseg = c->plan.nseg; p->vec = c->plan.vec;
+    p->segs_per_block = c->plan.segs_per_block; p->slots_per_block = c->plan.slots;
+    p->use_lds_reduce = c->plan.lds_reduce; p->fused_select = fused_select ? 1u : 0u;
+    return 0;
+}
+
+int check_dec_call(const Config* c, int dtype, uint32_t in_features, uint32_t out_features,
+                   const void* input, const void* output) {
+    DD_CHECK(c != nullptr, "invalid DECConfig handle");
+    DD_CHECK(input && output, "input and output pointers must not be null");
+    DD_CHECK(dtype == c->dt, "Mismatched data types between input tensor and DECConfig.");
+    DD_CHECK(in_features == c->K, "input tensor size does not match with DECConfig: input size: %u, DECConfig size: %u",
+             in_features, c->K);
+    DD_CHECK(out_features == c->N, "output tensor size does not match with DECConfig: output size: %u, DECConfig size: %u",
+             out_features, c->N);
+    DD_CHECK(c->ctx != nullptr && c->ctx->dt == c->dt, "Data type mismatch between DECConfig and DECContext.");
+    return kOk;
+}
+
+// ---- base-GEMV launch plans ------------------------------------------------------------------------
+struct AnyprecPlan { AnyprecParams p; LaunchDims d; };
+
+int plan_anyprec(const void* input, void* output, const void* qweight, const void* lut, int bits, int dtype,
+                 uint32_t K, uint32_t N, bool fused_block, AnyprecPlan* pl) {
+    DD_CHECK(bits >= 3 && bits <= 8, "Bitwidth must be between 3 and 8.");
+    if (dtype == DECDEC_FP32)
+        return fail(kUnsupported, "Any-Precision GEMV does not support float data type. Please use half or bfloat16.");
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(input && output && qweight && lut, "null pointer argument");
+    DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
+    DD_CHECK(N >= 1, "output_feat must be positive");
+    DD_CHECK(((uintptr_t)lut % 16) == 0 || bits != 3, "lut must be 16-byte aligned");
+    DD_CHECK(((uintptr_t)output % 4) == 0, "output must be 4-byte aligned");
+    AnyprecParams& p = pl->p;
+    memset(&p, 0, sizeof(p));
+    p.x = input; p.qweight = (const uint32_t*)qweight; p.lut = lut; p.out = output;
+    p.N = N; p.K = K; p.W = K / 32;
+    const uint32_t s_total = cdiv(p.W, 64);
+    p.sgroups = cdiv(s_total, 16);
+    p.S = cdiv(s_total, p.sgroups);
+    p.rg = fused_block ? std::max(1u, 16u / p.S) : std::max(1u, 8u / p.S);
+    uint32_t rpw = g_opt.anyprec_rpw > 0 ? (uint32_t)g_opt.anyprec_rpw
+                                         : (uint32_t)(((uint64_t)N * p.S * p.sgroups) / 2048);
+    rpw = std::min(16u, std::max(2u, rpw));
+    rpw += rpw & 1u;
+    p.rpw = rpw;
+    p.x_aligned = ((uintptr_t)input % 16) == 0;
+    pl->d.grid = cdiv(N, p.rg * p.rpw) * p.sgroups;
+    pl->d.block = fused_block ? 1024u : 64u * p.S * p.rg;
+    pl->d.lds = anyprec_lds_bytes(p.S, p.rg, p.rpw, bits);
+    return kOk;
+}
+
+struct LutgemmPlan { LutgemmParams p; LaunchDims d; };
+
+int plan_lutgemm(const void* input, void* output, const void* qw, const void* alpha, const void* q_bias, int bits,
+                 int group_size, int dtype, uint32_t K, uint32_t N, bool fused_block, LutgemmPlan* pl) {
+    DD_CHECK(bits >= 1 && bits <= 8, "Bitwidth must be between 1 and 8.");
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
+    DD_CHECK(input && output && qw && alpha && q_bias, "null pointer argument");
+    DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
+    DD_CHECK(group_size >= 32 && group_size % 32 == 0 && K % (uint32_t)group_size == 0,
+             "group_size must be a multiple of 32 that divides input_feat, got %d", group_size);
+    DD_CHECK(N >= 1, "output_feat must be positive");
+    LutgemmParams& p = pl->p;
+    memset(&p, 0, sizeof(p));
+    p.x = input; p.qw = (const uint32_t*)qw; p.alpha = alpha; p.q_bias = q_bias; p.out = output;
+    p.N = N; p.K = K; p.bits = (uint32_t)bits; p.group_size = (uint32_t)group_size;
+    p.ktb = std::min((uint32_t)kLutgemmMaxKtb, K / 32);
+    p.k_tiles = cdiv(K / 32, p.ktb);
+    const uint32_t threads = fused_block ? 1024u : 256u;
+    uint32_t npb = g_opt.lutgemm_npb > 0 ? (uint32_t)g_opt.lutgemm_npb : (fused_block ? 2048u : 1024u);
+    npb = std::max(2u * threads, npb);               // at least one output pair per thread
+    npb += npb & 1u;
+    p.npb = npb;
+    p.n_tiles = cdiv(N, npb);
+    pl->d.grid = p.n_tiles * p.k_tiles;
+    pl->d.block = threads;
+    pl->d.lds = lutgemm_lds_bytes(p.ktb);
+    return kOk;
+}
+
+struct SqllmPlan { SqllmParams p; LaunchDims d; };
+
+int plan_sqllm(const void* input, void* output, const void* mat, const void* lut, int bits, int dtype,
+               uint32_t K, uint32_t N, bool fused_block, SqllmPlan* pl) {
+    DD_CHECK(bits == 3 || bits == 4, "Bitwidth must be 3 or 4.");
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
+    DD_CHECK(input && output && mat && lut, "null pointer argument");
+    DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
+    DD_CHECK(N >= 1, "output_feat must be positive");
+    SqllmParams& p = pl->p;
+    memset(&p, 0, sizeof(p));
+    p.x = input; p.mat = (const uint32_t*)mat; p.lut = lut; p.out = output;
+    p.N = N; p.K = K; p.bits = (uint32_t)bits;
+    p.nthreads = 256;
+    p.n_tiles = cdiv(N, p.nthreads);
+    uint32_t kt = g_opt.sqllm_ktiles > 0 ? (uint32_t)g_opt.sqllm_ktiles : cdiv(2048, p.n_tiles);
+    kt = std::max(1u, std::min(kt, K / 128 ? K / 128 : 1u));
+    p.kspan = cdiv(cdiv(K, kt), 32) * 32;
+    p.k_tiles = cdiv(K, p.kspan);
+    pl->d.grid = p.n_tiles * p.k_tiles;
+    pl->d.block = fused_block ? 1024u : p.nthreads;
+    pl->d.lds = sqllm_lds_bytes(p.nthreads, p.bits, p.kspan);
+    return kOk;
+}
+
+// Side stream and events of the dummy_* calls (the reference creates and leaks a stream and two events
+// per call, decdec.cu:851-857; one set is enough).
+hipStream_t g_dummy_stream = nullptr;
+hipEvent_t g_dummy_e1 = nullptr, g_dummy_e2 = nullptr;
+
+int ensure_dummy_stream() {
+    if (!g_dummy_stream) {
+        DD_HIP(hipStreamCreateWithFlags(&g_dummy_stream, hipStreamNonBlocking));
+        DD_HIP(hipEventCreateWithFlags(&g_dummy_e1, hipEventDisableTiming));
+        DD_HIP(hipEventCreateWithFlags(&g_dummy_e2, hipEventDisableTiming));
+    }
+    return kOk;
+}
+
+// Two-stream form (reference decdec.cu:621-640): DEC on the caller's stream, the GEMV on the
+// context's sub-stream, joined by events.
+template <typename GemvLaunch>
+static int two_stream(Config* c, const DecParams* dp, bool have_dec, int dtype, hipStream_t main_stream,
+                      GemvLaunch gemv) {
+    hipStream_t sub = c->ctx->sub_stream;
+    DD_HIP(hipEventRecord(c->e1, main_stream));
+    if (have_dec) {
+        LaunchDims d{c->plan.cg * c->plan.sg, (uint32_t)kDecThreads, c->plan.lds};
+        DD_HIP(launch_dec(dtype, *dp, d, main_stream));
+    }
+    DD_HIP(hipStreamWaitEvent(sub, c->e1, 0));
+    DD_HIP(gemv(sub));
+    DD_HIP(hipEventRecord(c->e2, sub));
+    DD_HIP(hipStreamWaitEvent(main_stream, c->e2, 0));
+    return kOk;
+}
+
+template <typename GemvLaunch>
+static int dummy_common(int dummy_cu, int64_t iters, hipStream_t main_stream, GemvLaunch gemv) {
+    int rc = ensure_dummy_stream();
+    if (rc != kOk) return rc;
+    DD_HIP(hipEventRecord(g_dummy_e1, main_stream));
+    if (dummy_cu > 0) DD_HIP(launch_burner((uint32_t)dummy_cu, (long long)iters, main_stream));
+    DD_HIP(hipStreamWaitEvent(g_dummy_stream, g_dummy_e1, 0));
+    DD_HIP(gemv(g_dummy_stream));
+    DD_HIP(hipEventRecord(g_dummy_e2, g_dummy_stream));
+    DD_HIP(hipStreamWaitEvent(main_stream, g_dummy_e2, 0));
+    return kOk;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* decdec_last_error(void) { return g_error.c_str(); }
+int decdec_version(void) { return 100; }
+
+int decdec_set_option(const char* name, int value) {
+    int* s = option_slot(name);
+    DD_CHECK(s != nullptr, "unknown option '%s'", name ? name : "(null)");
+    *s = value;
+    return kOk;
+}
+int decdec_get_option(const char* name, int* value) {
+    int* s = option_slot(name);
+    DD_CHECK(s != nullptr && value != nullptr, "unknown option '%s'", name ? name : "(null)");
+    *value = *s;
+    return kOk;
+}
+
+int decdec_bucket_floors(float a, float b, int dtype, float* out) {
+    DD_CHECK(dtype_ok(dtype) && out, "invalid argument");
+    bucket_floors(round_to(a, dtype), round_to(b, dtype), dtype, out);
+    return kOk;
+}
+
+int decdec_reference_geometry(uint32_t K, uint32_t N, uint32_t n_tb, uint32_t k_chunk, int dtype,
+                              uint32_t max_smem, decdec_config_info* out) {
+    DD_CHECK(dtype_ok(dtype) && out && n_tb >= 1 && N >= 8, "invalid argument");
+    memset(out, 0, sizeof(*out));
+    const int st = reference_geometry(K, N, n_tb, k_chunk, dtype, max_smem, out);
+    DD_CHECK(st != 1, "output size too small");
+    return kOk;
+}
+
+// ---------------------------------------------------------------- context
+int decdec_create_dec_context(uint32_t num_tb, int dtype, uint64_t buffer_numel, void* rows, void* acts,
+                              uint64_t* out) {
+    DD_CHECK(out != nullptr, "context_out must not be null");
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
+    DD_CHECK(rows != nullptr && acts != nullptr, "selected_rows_buffer and selected_activations_buffer must be on GPU.");
+    DD_CHECK(num_tb >= 1, "num_tb must be at least 1");
+    Context* c = new Context();
+    c->dt = dtype; c->num_tb = num_tb; c->buffer_numel = buffer_numel;
+    c->rows = (int32_t*)rows; c->acts = acts; c->sub_stream = nullptr; c->event = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&c->sub_stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->event, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        if (c->sub_stream) (void)hipStreamDestroy(c->sub_stream);
+        delete c;
+        return fail(kHipError, "HIP error creating the DEC context: %s", hipGetErrorString(e));
+    }
+    {
+        std::lock_guard<std::mutex> l(g_mu);
+        g_contexts.insert(reinterpret_cast<uint64_t>(c));
+    }
+    *out = reinterpret_cast<uint64_t>(c);
+    return kOk;
+}
+
+int decdec_destroy_dec_context(uint64_t h) {
+    Context* c = get_context(h);
+    DD_CHECK(c != nullptr, "invalid DECContext handle");
+    {
+        std::lock_guard<std::mutex> l(g_mu);
+        g_contexts.erase(h);
+    }
+    (void)hipStreamDestroy(c->sub_stream);
+    (void)hipEventDestroy(c->event);
+    delete c;
+    return kOk;
+}
+
+// ---------------------------------------------------------------- config
+int decdec_create_dec_config(uint64_t ctx_h, uint32_t k_chunk, int dtype, const void* q_residual,
+                             int q_on_device, const void* scales, int scales_on_device,
+                             const void* thresholds_host, uint32_t num_rows, uint32_t num_cols, uint64_t* out) {
+    Context* ctx = get_context(ctx_h);
+    DD_CHECK(ctx != nullptr, "invalid DECContext handle");
+    DD_CHECK(out != nullptr, "config_out must not be null");
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type in create_dec_config.");
+    DD_CHECK(dtype == ctx->dt, "Data type mismatch between DECConfig and DECContext.");
+    DD_CHECK(q_residual && scales && thresholds_host, "null pointer argument");
+    DD_CHECK(num_rows >= 1 && num_cols >= 8 && num_cols % 8 == 0,
+             "q_residual must be [in_features, out_features / 8] with out_features a multiple of 8");
+    Config* c = new Config();
+    memset(c, 0, sizeof(*c));
+    c->dt = dtype; c->ctx = ctx; c->K = num_rows; c->N = num_cols; c->M = num_cols / 8;
+    c->thresholds_host = thresholds_host;
+    int dev = 0, smem = 65536;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&smem, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+    const size_t res_bytes = (size_t)num_rows * c->M * 4, sc_bytes = (size_t)num_cols * dtype_size(dtype);
+    if (e == hipSuccess) {
+        c->max_smem = (uint32_t)smem;
+        if (q_on_device) {
+            fprintf(stderr, "DecDEC WARNING: q_residual is on the GPU; it is used in place and zero-copy host memory is NOT used.\n");
+            c->residual_dev = (const uint32_t*)q_residual;
+        } else {
+            unsigned flags = hipHostMallocMapped | (g_opt.host_noncoherent ? hipHostMallocNonCoherent : 0u);
+            e = hipHostMalloc(&c->residual_host, res_bytes, flags);
+            if (e == hipSuccess) {
+                memcpy(c->residual_host, q_residual, res_bytes);
+                void* d = nullptr;
+                e = hipHostGetDevicePointer(&d, c->residual_host, 0);
+                c->residual_dev = (const uint32_t*)d;
+            }
+        }
+    }
+    if (e == hipSuccess) e = hipMalloc(&c->scales_dev, sc_bytes);
+    if (e == hipSuccess)
+        e = hipMemcpy(c->scales_dev, scales, sc_bytes, scales_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->e1, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->e2, hipEventDisableTiming);
+    int rc = kOk;
+    if (e != hipSuccess) rc = fail(kHipError, "HIP error in create_dec_config: %s", hipGetErrorString(e));
+    if (rc == kOk) rc = setup_config(c, k_chunk);
+    if (rc != kOk) {
+        if (c->residual_host) (void)hipHostFree(c->residual_host);
+        if (c->scales_dev) (void)hipFree(c->scales_dev);
+        if (c->e1) (void)hipEventDestroy(c->e1);
+        if (c->e2) (void)hipEventDestroy(c->e2);
+        delete c;
+        return rc;
+    }
+    {
+        std::lock_guard<std::mutex> l(g_mu);
+        g_configs.insert(reinterpret_cast<uint64_t>(c));
+    }
+    *out = reinterpret_cast<uint64_t>(c);
+    return kOk;
+}
+
+int decdec_read_dec_config(uint64_t h, decdec_config_info* info) {
+    Config* c = get_config(h);
+    DD_CHECK(c != nullptr && info != nullptr, "invalid DECConfig handle");
+    *info = c->info;
+    return kOk;
+}
+
+int decdec_update_dec_config(uint64_t h, uint64_t new_ctx, uint32_t k_chunk) {
+    Config* c = get_config(h);
+    DD_CHECK(c != nullptr, "invalid DECConfig handle");
+    Context* ctx = get_context(new_ctx);
+    DD_CHECK(ctx != nullptr, "invalid DECContext handle");
+    DD_CHECK(ctx->dt == c->dt, "Data type mismatch between DECConfig and DECContext.");
+    Context* old = c->ctx;
+    const uint32_t old_k = c->k_chunk;
+    c->ctx = ctx;
+    const int rc = setup_config(c, k_chunk);
+    if (rc != kOk) {
+        const std::string msg = g_error;
+        c->ctx = old;
+        (void)setup_config(c, old_k);
+        g_error = msg;
+        return rc;
+    }
+    return kOk;
+}
+
+int decdec_destroy_dec_config(uint64_t h) {
+    Config* c = get_config(h);
+    DD_CHECK(c != nullptr, "invalid DECConfig handle");
+    {
+        std::lock_guard<std::mutex> l(g_mu);
+        g_configs.erase(h);
+    }
+    if (c->residual_host) (void)hipHostFree(c->residual_host);
+    if (c->scales_dev) (void)hipFree(c->scales_dev);
+    (void)hipEventDestroy(c->e1);
+    (void)hipEventDestroy(c->e2);
+    delete c;
+    return kOk;
+}
+
+// ---------------------------------------------------------------- DEC
+static int dec_common(uint64_t h, const void* input, void* output, int dtype, uint32_t K, uint32_t N,
+                      void* stream, bool fused_select) {
+    Config* c = get_config(h);
+    int rc = check_dec_call(c, dtype, K, N, input, output);
+    if (rc != kOk) return rc;
+    DecParams p;
+    if (fill_dec_params(c, input, output, fused_select, &p)) return kOk;
+    LaunchDims d{c->plan.cg * c->plan.sg, (uint32_t)kDecThreads, c->plan.lds};
+    DD_HIP(launch_dec(dtype, p, d, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_dec(uint64_t h, const void* input, void* output, int dtype, uint32_t K, uint32_t N, void* stream) {
+    return dec_common(h, input, output, dtype, K, N, stream, true);
+}
+int decdec_unfused_dec(uint64_t h, const void* input, void* output, int dtype, uint32_t K, uint32_t N, void* stream) {
+    return dec_common(h, input, output, dtype, K, N, stream, false);
+}
+
+// ---------------------------------------------------------------- base GEMVs
+int decdec_anyprec_gemv(const void* input, void* output, const void* qweight, const void* lut, int bits,
+                        int dtype, uint32_t K, uint32_t N, void* stream) {
+    AnyprecPlan pl;
+    int rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    DD_HIP(launch_anyprec(dtype, bits, pl.p, pl.d, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_anyprec_dequant(const void* qweight, const void* lut, void* weight, int bits, int dtype,
+                           uint32_t N, uint32_t K, void* stream) {
+    DD_CHECK(bits >= 3 && bits <= 8, "Bitwidth must be between 3 and 8.");
+    if (dtype == DECDEC_FP32)
+        return fail(kUnsupported, "Any-Precision Dequantization does not support float data type. Please use half or bfloat16.");
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(qweight && lut && weight, "null pointer argument");
+    DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
+    DD_HIP(launch_anyprec_dequant(dtype, bits, (const uint32_t*)qweight, lut, weight, N, K, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_lutgemm_gemv(const void* input, void* output, const void* qw, const void* alpha, const void* q_bias,
+                        int bits, int group_size, int dtype, uint32_t K, uint32_t N, void* stream) {
+    LutgemmPlan pl;
+    int rc = plan_lutgemm(input, output, qw, alpha, q_bias, bits, group_size, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    DD_HIP(launch_lutgemm(dtype, pl.p, pl.d, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_sqllm_gemv(const void* input, void* output, const void* mat, const void* lut, int bits, int dtype,
+                      uint32_t K, uint32_t N, void* stream) {
+    SqllmPlan pl;
+    int rc = plan_sqllm(input, output, mat, lut, bits, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    DD_HIP(launch_sqllm(dtype, pl.p, pl.d, (hipStream_t)stream));
+    return kOk;
+}
+
+// ---------------------------------------------------------------- DEC + base GEMV
+int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
+                       int bits, int dtype, uint32_t K, uint32_t N, void* stream) {
+    Config* c = get_config(h);
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    int rc = check_dec_call(c, dtype, K, N, input, output);
+    if (rc != kOk) return rc;
+    DecParams dp;
+    const bool have_dec = fill_dec_params(c, input, output, true, &dp) == 0;
+    const bool fuse = g_opt.fusion && have_dec;
+    AnyprecPlan pl;
+    rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, fuse, &pl);
+    if (rc != kOk) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (fuse) {
+        LaunchDims d = pl.d;
+        d.lds = std::max(d.lds, c->plan.lds);
+        DD_HIP(launch_dec_anyprec(dtype, bits, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        return kOk;
+    }
+    if (!have_dec && g_opt.fusion) { DD_HIP(launch_anyprec(dtype, bits, pl.p, pl.d, s)); return kOk; }
+    return two_stream(c, &dp, have_dec, dtype, s,
+                      [&](hipStream_t sub) { return launch_anyprec(dtype, bits, pl.p, pl.d, sub); });
+}
+
+int decdec_dec_lutgemm(uint64_t h, const void* input, void* output, const void* qw, const void* alpha,
+                       const void* q_bias, int bits, int group_size, int dtype, uint32_t K, uint32_t N,
+                       void* stream) {
+    Config* c = get_config(h);
+    int rc = check_dec_call(c, dtype, K, N, input, output);
+    if (rc != kOk) return rc;
+    DecParams dp;
+    const bool have_dec = fill_dec_params(c, input, output, true, &dp) == 0;
+    const bool fuse = g_opt.fusion && have_dec;
+    LutgemmPlan pl;
+    rc = plan_lutgemm(input, output, qw, alpha, q_bias, bits, group_size, dtype, K, N, fuse, &pl);
+    if (rc != kOk) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (fuse) {
+        LaunchDims d = pl.d;
+        d.lds = std::max(d.lds, c->plan.lds);
+        DD_HIP(launch_dec_lutgemm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        return kOk;
+    }
+    if (!have_dec && g_opt.fusion) { DD_HIP(launch_lutgemm(dtype, pl.p, pl.d, s)); return kOk; }
+    return two_stream(c, &dp, have_dec, dtype, s, [&](hipStream_t sub) { return launch_lutgemm(dtype, pl.p, pl.d, sub); });
+}
+
+int decdec_dec_sqllm(uint64_t h, const void* input, void* output, const void* mat, const void* lut, int bits,
+                     int dtype, uint32_t K, uint32_t N, void* stream) {
+    Config* c = get_config(h);
+    int rc = check_dec_call(c, dtype, K, N, input, output);
+    if (rc != kOk) return rc;
+    DecParams dp;
+    const bool have_dec = fill_dec_params(c, input, output, true, &dp) == 0;
+    const bool fuse = g_opt.fusion && have_dec;
+    SqllmPlan pl;
+    rc = plan_sqllm(input, output, mat, lut, bits, dtype, K, N, fuse, &pl);
+    if (rc != kOk) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (fuse) {
+        LaunchDims d = pl.d;
+        d.lds = std::max(d.lds, c->plan.lds);
+        DD_HIP(launch_dec_sqllm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        return kOk;
+    }
+    if (!have_dec && g_opt.fusion) { DD_HIP(launch_sqllm(dtype, pl.p, pl.d, s)); return kOk; }
+    return two_stream(c, &dp, have_dec, dtype, s, [&](hipStream_t sub) { return launch_sqllm(dtype, pl.p, pl.d, sub); });
+}
+
+// ---------------------------------------------------------------- dummies
+int decdec_dummy_anyprec(const void* input, void* output, const void* qweight, const void* lut, int bits,
+                         int dtype, uint32_t K, uint32_t N, int dummy_cu, int64_t iters, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "dummy_anyprec supports FP16/BF16 only.");
+    AnyprecPlan pl;
+    int rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    return dummy_common(dummy_cu, iters, (hipStream_t)stream,
+                        [&](hipStream_t sub) { return launch_anyprec(dtype, bits, pl.p, pl.d, sub); });
+}
+
+int decdec_dummy_lutgemm(const void* input, void* output, const void* qw, const void* alpha, const void* q_bias,
+                         int bits, int group_size, int dtype, uint32_t K, uint32_t N, int dummy_cu,
+                         int64_t iters, void* stream) {
+    LutgemmPlan pl;
+    int rc = plan_lutgemm(input, output, qw, alpha, q_bias, bits, group_size, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    return dummy_common(dummy_cu, iters, (hipStream_t)stream,
+                        [&](hipStream_t sub) { return launch_lutgemm(dtype, pl.p, pl.d, sub); });
+}
+
+int decdec_dummy_sqllm(const void* input, void* output, const void* mat, const void* lut, int bits, int dtype,
+                       uint32_t K, uint32_t N, int dummy_cu, int64_t iters, void* stream) {
+    DD_CHECK(bits == 3 || bits == 4, "SQLLM bitwidth must be 3 or 4.");
+    SqllmPlan pl;
+    int rc = plan_sqllm(input, output, mat, lut, bits, dtype, K, N, false, &pl);
+    if (rc != kOk) return rc;
+    return dummy_common(dummy_cu, iters, (hipStream_t)stream,
+                        [&](hipStream_t sub) { return launch_sqllm(dtype, pl.p, pl.d, sub); });
+}
+
+}  // extern "C"

@@ -1,0 +1,102 @@
+// Any-precision bitplane kernels: GEMV, dequantisation to a dense [N, K] matrix, and the fused
+// single-launch DEC + GEMV kernel.
+#include "launch.h"
+
+namespace decdec {
+
+template <int DT, int BITS>
+__global__ __launch_bounds__(1024) void anyprec_kernel(const AnyprecParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    anyprec_role<DT, BITS>(p, blockIdx.x, smem);
+}
+
+template <int DT, int BITS>
+__global__ __launch_bounds__(1024) void dec_anyprec_kernel(const DecParams dp, const uint32_t dec_blocks,
+                                                           const AnyprecParams gp) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
+    else anyprec_role<DT, BITS>(gp, blockIdx.x - dec_blocks, smem);
+}
+
+// W[n][c] = lut[n][idx(n, c)]: one thread per (row, word); the 32 weights of a word go to four groups
+// of eight consecutive channels (reference dequant_kbit_store, decdec_extension/anyprec.cu:261-331).
+template <int DT, int BITS>
+__global__ __launch_bounds__(256) void anyprec_dequant_kernel(const uint32_t* __restrict__ qweight,
+                                                              const void* __restrict__ lut, void* __restrict__ weight,
+                                                              const uint32_t N, const uint32_t K) {
+    const uint32_t W = K / 32u;
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (size_t)N * W) return;
+    const uint32_t n = (uint32_t)(gid / W), wi = (uint32_t)(gid % W);
+    const uint32_t i = wi >> 5, t = wi & 31u;
+    const uint32_t eff = (i == K / 1024u) ? (K % 1024u) / 32u : 32u;
+    uint32_t q[BITS];
+#pragma unroll
+    for (int pl = 0; pl < BITS; ++pl) q[pl] = qweight[((size_t)pl * N + n) * W + wi];
+    constexpr int L = 1 << BITS;
+    const uint16_t* lrow = (const uint16_t*)lut + (size_t)n * L;
+    uint16_t* wrow = (uint16_t*)weight + (size_t)n * K;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint16_t vals[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int pos = 31 - (8 * j + e);
+            uint32_t idx = 0;
+#pragma unroll
+            for (int pl = 0; pl < BITS; ++pl) idx = (idx << 1) | ((q[pl] >> pos) & 1u);
+            vals[e] = lrow[idx];
+        }
+        uint16_t* dst = wrow + (size_t)1024 * i + (size_t)8 * eff * j + (size_t)8 * t;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[e] = vals[e];
+    }
+}
+
+#define DD_BITS_SWITCH(BITS_EXPR, CALL)                \
+    switch (BITS_EXPR) {                               \
+        case 3: { constexpr int B = 3; CALL; } break;  \
+        case 4: { constexpr int B = 4; CALL; } break;  \
+        case 5: { constexpr int B = 5; CALL; } break;  \
+        case 6: { constexpr int B = 6; CALL; } break;  \
+        case 7: { constexpr int B = 7; CALL; } break;  \
+        case 8: { constexpr int B = 8; CALL; } break;  \
+        default: return hipErrorInvalidValue;          \
+    }
+
+hipError_t launch_anyprec(int dt, int bits, const AnyprecParams& p, const LaunchDims& d, hipStream_t s) {
+    if (dt == kFP16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((anyprec_kernel<kFP16, B>), dim3(d.grid), dim3(d.block), d.lds, s, p));
+    } else if (dt == kBF16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((anyprec_kernel<kBF16, B>), dim3(d.grid), dim3(d.block), d.lds, s, p));
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t dec_blocks,
+                              const AnyprecParams& gp, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(dec_blocks + d.grid), block(d.block);
+    if (dt == kFP16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kFP16, B>), grid, block, d.lds, s, dp, dec_blocks, gp));
+    } else if (dt == kBF16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, B>), grid, block, d.lds, s, dp, dec_blocks, gp));
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_anyprec_dequant(int dt, int bits, const uint32_t* qweight, const void* lut, void* weight,
+                                  uint32_t N, uint32_t K, hipStream_t s) {
+    const size_t total = (size_t)N * (K / 32u);
+    const dim3 grid((uint32_t)((total + 255) / 256)), block(256);
+    if (total == 0) return hipSuccess;
+    // 16-bit LUT entries are copied bit for bit, so fp16 and bf16 share one instantiation
+    if (dt != kFP16 && dt != kBF16) return hipErrorInvalidValue;
+    DD_BITS_SWITCH(bits, hipLaunchKernelGGL((anyprec_dequant_kernel<kFP16, B>), grid, block, 0, s, qweight, lut, weight, N, K));
+    return hipGetLastError();
+}
+
+}  // namespace decdec

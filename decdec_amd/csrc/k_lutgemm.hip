@@ -1,0 +1,42 @@
+// LUT-GEMM kernels: GEMV and the fused single-launch DEC + GEMV kernel.
+#include "launch.h"
+
+namespace decdec {
+
+template <int DT>
+__global__ __launch_bounds__(1024) void lutgemm_kernel(const LutgemmParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    lutgemm_role<DT>(p, blockIdx.x, smem);
+}
+
+template <int DT>
+__global__ __launch_bounds__(1024) void dec_lutgemm_kernel(const DecParams dp, const uint32_t dec_blocks,
+                                                           const LutgemmParams gp) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
+    else lutgemm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
+}
+
+hipError_t launch_lutgemm(int dt, const LutgemmParams& p, const LaunchDims& d, hipStream_t s) {
+    switch (dt) {
+        case kFP32: hipLaunchKernelGGL(lutgemm_kernel<kFP32>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        case kFP16: hipLaunchKernelGGL(lutgemm_kernel<kFP16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        case kBF16: hipLaunchKernelGGL(lutgemm_kernel<kBF16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
+                              const LutgemmParams& gp, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(dec_blocks + d.grid), block(d.block);
+    switch (dt) {
+        case kFP32: hipLaunchKernelGGL(dec_lutgemm_kernel<kFP32>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kFP16: hipLaunchKernelGGL(dec_lutgemm_kernel<kFP16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kBF16: hipLaunchKernelGGL(dec_lutgemm_kernel<kBF16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace decdec

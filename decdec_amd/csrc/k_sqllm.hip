@@ -1,0 +1,42 @@
+// SqueezeLLM kernels: GEMV and the fused single-launch DEC + GEMV kernel.
+#include "launch.h"
+
+namespace decdec {
+
+template <int DT>
+__global__ __launch_bounds__(1024) void sqllm_kernel(const SqllmParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    sqllm_role<DT>(p, blockIdx.x, smem);
+}
+
+template <int DT>
+__global__ __launch_bounds__(1024) void dec_sqllm_kernel(const DecParams dp, const uint32_t dec_blocks,
+                                                           const SqllmParams gp) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
+    else sqllm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
+}
+
+hipError_t launch_sqllm(int dt, const SqllmParams& p, const LaunchDims& d, hipStream_t s) {
+    switch (dt) {
+        case kFP32: hipLaunchKernelGGL(sqllm_kernel<kFP32>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        case kFP16: hipLaunchKernelGGL(sqllm_kernel<kFP16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        case kBF16: hipLaunchKernelGGL(sqllm_kernel<kBF16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
+                              const SqllmParams& gp, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(dec_blocks + d.grid), block(d.block);
+    switch (dt) {
+        case kFP32: hipLaunchKernelGGL(dec_sqllm_kernel<kFP32>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kFP16: hipLaunchKernelGGL(dec_sqllm_kernel<kFP16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kBF16: hipLaunchKernelGGL(dec_sqllm_kernel<kBF16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace decdec

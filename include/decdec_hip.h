@@ -1,0 +1,155 @@
+/*
+ * C ABI of libdecdec_hip.so -- the MI355X (gfx950) implementation of DecDEC's decode-time
+ * linear-layer path.  Plain pointers and sizes only; no torch types.
+ *
+ * Every entry point replaces one function of the reference's pybind module `decdec_ext`
+ * (reference decdec_extension/bindings.cpp:19-40); the reference function and the file:line of
+ * its C++ implementation are cited at each declaration.  Tensor arguments of the reference become
+ * (pointer, dtype, sizes); the "current CUDA stream" of the reference (decdec.cu:144, :331)
+ * becomes the explicit `stream` argument (a hipStream_t; NULL = default stream).
+ *
+ * Conventions
+ *   - return value 0 = success; non-zero = failure, decdec_last_error() then returns a message
+ *     (thread-local).  1 = invalid argument, 2 = HIP runtime error, 3 = unsupported.
+ *   - all device pointers must be valid on the current HIP device; kernels are enqueued on
+ *     `stream` and the calls do not synchronise.
+ *   - every GEMV / DEC entry point ACCUMULATES into `output` with atomic adds, as the reference
+ *     kernels do (anyprec.cu:508-510, lutgemm.cu:143-148, sqllm.cu:115, dec.cu:275): callers
+ *     zero `output` first (reference end-to-end/APLinear.py:51).
+ *   - handles are opaque 64-bit integers (the reference returns uintptr_t object addresses,
+ *     dec_config.cu:243, dec_context.cu:59).
+ *   - not thread-safe per handle; callers are single-threaded like the reference's.
+ */
+#ifndef DECDEC_HIP_H
+#define DECDEC_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of activations / scales / LUTs / outputs (reference datatype.h:8-12) */
+enum { DECDEC_FP32 = 0, DECDEC_FP16 = 1, DECDEC_BF16 = 2 };
+
+typedef struct decdec_config_info {
+    /* keys of the reference's read_dec_config (dec_config.cu:343-351), computed with the
+     * reference's own integer formulas (dec_config.cu:34-115) so tools that read them see the
+     * same values */
+    int32_t num_chunks, chunk_size, k_chunk, channels_per_tb, n_tb;
+    int32_t block_dim_x, block_dim_y, shared_memory_size, reduced_shared_memory;
+    /* launch plan actually used by the gfx950 DEC kernel */
+    int32_t hip_dec_blocks;        /* workgroups of 1024 threads given to DEC (<= num_tb) */
+    int32_t hip_chunk_groups;      /* = atomic adds each output receives from DEC */
+    int32_t hip_segment_groups;
+    int32_t hip_vec_words;         /* u32 words per lane per residual load: 1, 2, 4 */
+    int32_t hip_lds_bytes;
+    int32_t hip_slots_per_block;
+    int32_t hip_lds_reduce;
+    int32_t hip_residual_on_host;  /* 1: zero-copy from pinned host memory */
+} decdec_config_info;
+
+const char* decdec_last_error(void);
+int decdec_version(void);
+
+/* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
+ * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
+ * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "lutgemm_npb",
+ * "sqllm_ktiles" (launch-shape overrides, 0 = automatic).  No counterpart in the reference. */
+int decdec_set_option(const char* name, int value);
+int decdec_get_option(const char* name, int* value);
+
+/* create_dec_context (dec_context.cu:62-103).  Borrows the two scratch buffers (device memory,
+ * `buffer_numel` elements each: int32 rows, `dtype` activations); creates the sub-stream and event
+ * used by the two-stream mode.  The reference has no destroy; decdec_destroy_dec_context is an
+ * addition. */
+int decdec_create_dec_context(uint32_t num_tb, int dtype, uint64_t buffer_numel,
+                              void* selected_rows_buffer, void* selected_activations_buffer,
+                              uint64_t* context_out);
+int decdec_destroy_dec_context(uint64_t context);
+
+/* create_dec_config (dec_config.cu:186-292).  q_residual: int32 [num_rows, num_cols/8]; when it is
+ * host memory it is copied into pinned, device-mapped memory owned by the config (zero-copy fetch);
+ * when it is device memory it is used in place (borrowed).  reordered_scales: `dtype`[num_cols],
+ * copied into device memory owned by the config.  thresholds: host memory, `dtype`[num_rows],
+ * BORROWED -- read again at every decdec_dec* call (decdec.cu:66-67), so it must outlive the config. */
+int decdec_create_dec_config(uint64_t context, uint32_t k_chunk, int dtype,
+                             const void* q_residual, int q_residual_on_device,
+                             const void* reordered_scales, int reordered_scales_on_device,
+                             const void* thresholds_host,
+                             uint32_t num_rows, uint32_t num_cols, uint64_t* config_out);
+/* read_dec_config (dec_config.cu:337-354) */
+int decdec_read_dec_config(uint64_t config, decdec_config_info* info_out);
+/* update_dec_config (dec_config.cu:295-326): new context and k_chunk, residual not re-copied */
+int decdec_update_dec_config(uint64_t config, uint64_t new_context, uint32_t k_chunk);
+/* destroy_dec_config (dec_config.cu:329-334) */
+int decdec_destroy_dec_config(uint64_t config);
+
+/* dec (decdec.cu:139-146 -> dec_templated :40-91 -> fused_dec_kernel dec.cu:26-280): select
+ * k_chunk channels per 1024-channel chunk, fetch their residual rows, accumulate into output.
+ * Writes the selection into the context's scratch buffers at [chunk*k_chunk + pos]. */
+int decdec_dec(uint64_t config, const void* input, void* output, int dtype,
+               uint32_t in_features, uint32_t out_features, void* stream);
+/* unfused_dec (decdec.cu:238-245 -> dec_kernel dec.cu:284-426): as dec, but the first
+ * k_chunk*in_features/1024 entries of the context's row buffer are supplied by the caller. */
+int decdec_unfused_dec(uint64_t config, const void* input, void* output, int dtype,
+                       uint32_t in_features, uint32_t out_features, void* stream);
+
+/* anyprec_gemv (decdec.cu:324-333 -> matmul_kbit_32 anyprec.cu:344-514). qweight int32
+ * [>=bitwidth, out, in/32] (only the first `bitwidth` planes are read; `qweight_planes` is the
+ * allocated plane count), lut `dtype`[out, 2^bitwidth]; fp16 / bf16 only; bitwidth 3..8. */
+int decdec_anyprec_gemv(const void* input, void* output, const void* qweight, const void* lut,
+                        int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
+                        void* stream);
+/* anyprec_dequant (decdec.cu:386-393 -> dequant_kbit_store anyprec.cu:261-331): weight_out
+ * `dtype`[out, in], allocated by the caller. */
+int decdec_anyprec_dequant(const void* qweight, const void* lut, void* weight_out, int bitwidth,
+                           int dtype, uint32_t out_features, uint32_t in_features, void* stream);
+/* lutgemm_gemv (decdec.cu:485-496 -> nqmv_bias lutgemm.cu:25-150). q_weight int32
+ * [in/32, bitwidth, out], alpha [in/group, bitwidth, out], q_bias [in/group, out]. */
+int decdec_lutgemm_gemv(const void* input, void* output, const void* q_weight, const void* alpha,
+                        const void* q_bias, int bitwidth, int group_size, int dtype,
+                        uint32_t in_features, uint32_t out_features, void* stream);
+/* sqllm_gemv (decdec.cu:594-603 -> VecQuant{3,4}MatMulKernelNUQPerChannel sqllm.cu:28-169).
+ * qweight int32 [in*bitwidth/32, out], lut [out, 2^bitwidth]; bitwidth 3 or 4. */
+int decdec_sqllm_gemv(const void* input, void* output, const void* qweight, const void* lut,
+                      int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
+                      void* stream);
+
+/* dec_anyprec / dec_lutgemm / dec_sqllm (decdec.cu:643-659, :701-721, :761-779): DEC and the base
+ * GEMV run concurrently on the pre-zeroed output; on return the work is ordered on `stream`. */
+int decdec_dec_anyprec(uint64_t config, const void* input, void* output, const void* qweight,
+                       const void* lut, int bitwidth, int dtype, uint32_t in_features,
+                       uint32_t out_features, void* stream);
+int decdec_dec_lutgemm(uint64_t config, const void* input, void* output, const void* q_weight,
+                       const void* alpha, const void* q_bias, int bitwidth, int group_size,
+                       int dtype, uint32_t in_features, uint32_t out_features, void* stream);
+int decdec_dec_sqllm(uint64_t config, const void* input, void* output, const void* qweight,
+                     const void* lut, int bitwidth, int dtype, uint32_t in_features,
+                     uint32_t out_features, void* stream);
+
+/* dummy_anyprec / dummy_lutgemm / dummy_sqllm (decdec.cu:874-1013): the base GEMV on a side stream
+ * while `dummy_cu` workgroups of 1024 threads spin for `dummy_iters` iterations on `stream`. */
+int decdec_dummy_anyprec(const void* input, void* output, const void* qweight, const void* lut,
+                         int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
+                         int dummy_cu, int64_t dummy_iters, void* stream);
+int decdec_dummy_lutgemm(const void* input, void* output, const void* q_weight, const void* alpha,
+                         const void* q_bias, int bitwidth, int group_size, int dtype,
+                         uint32_t in_features, uint32_t out_features,
+                         int dummy_cu, int64_t dummy_iters, void* stream);
+int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, const void* lut,
+                       int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
+                       int dummy_cu, int64_t dummy_iters, void* stream);
+
+/* Host-only helpers (no GPU needed).  decdec_bucket_floors evaluates the selector's 32 bucket
+ * floors exactly as dec.cu:117-130 does, in `dtype` arithmetic; decdec_reference_geometry evaluates
+ * dec_config.cu:34-115 for a shape.  No counterpart in the reference's API. */
+int decdec_bucket_floors(float threshold_a, float threshold_b, int dtype, float* floors32_out);
+int decdec_reference_geometry(uint32_t num_rows, uint32_t num_cols, uint32_t num_tb,
+                              uint32_t k_chunk, int dtype, uint32_t max_shared_memory,
+                              decdec_config_info* info_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DECDEC_HIP_H */

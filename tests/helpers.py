@@ -1,0 +1,40 @@
+"""Shared builders for the parity tests (synthetic layers in the benchmark's recipe)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from decdec_amd import formats as F
+
+TORCH_DT = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+def np_of(t: torch.Tensor) -> np.ndarray:
+    """Tensor -> numpy; bf16 goes through float32 (values stay exactly representable)."""
+    t = t.detach().cpu()
+    return t.float().numpy() if t.dtype == torch.bfloat16 else t.numpy()
+
+
+def make_dec_layer(K, N, seed, dtype=torch.float16, random_residual=False):
+    """Weights, quantised base (any-precision 3-bit) and 4-bit residual of one layer, on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    W = (torch.randn(N, K, generator=g) * 0.02).to(torch.float16)
+    idx, lut = F.quantize_uniform_rows(W, 3)
+    Wq = F.dequant_lut(idx, lut)
+    if random_residual:
+        cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32)
+        scales = torch.rand(N, generator=g)
+    else:
+        q, s = F.quantize_residual((W.float() - Wq.float()).to(torch.float16))
+        cheat, scales = F.pack_residual(q, s)
+    x = F.make_activation(K, g, dtype=dtype)
+    th = F.calibrate_thresholds(K, g, draws=16, dtype=dtype)
+    return {"W": W, "idx": idx, "lut": lut.to(dtype), "qweight": F.pack_anyprec(idx, 3),
+            "cheat": cheat.contiguous(), "scales": scales.to(dtype).contiguous(), "x": x, "th": th}
+
+
+def rel_err(got: np.ndarray, want: np.ndarray):
+    """(max relative error with a floor of 1e-2*max|want| in the denominator, mean abs error)."""
+    got = got.astype(np.float64); want = want.astype(np.float64)
+    denom = np.maximum(np.abs(want), 1e-2 * np.max(np.abs(want)) + 1e-30)
+    return float(np.max(np.abs(got - want) / denom)), float(np.mean(np.abs(got - want)))
