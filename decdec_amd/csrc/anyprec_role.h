@@ -29,7 +29,7 @@ struct AnyprecParams {
     uint32_t S;            // slices (waves) per row handled inside one workgroup (<= 16)
     uint32_t sgroups;      // slice groups (> 1 only when ceil(W/64) > 16, i.e. K > 32768)
     uint32_t rg;           // row groups per workgroup
-    uint32_t rpw;          // rows per wave (even)
+    uint32_t rpw;          // rows per wave: 2, 4 or 8, all in flight together
     uint32_t x_aligned;    // activation pointer is 16-byte aligned
 };
 
@@ -48,12 +48,12 @@ __device__ __forceinline__ float dot2_acc(uint32_t w, uint32_t x, float acc) {
     }
 }
 
-// Load the 32 activations that belong to word `wi` of a row, arranged for the decoders below:
+// The 32 activations that belong to word `wi` of a row: issue the loads (xr[j] = the eight 16-bit values
+// of group j), then arrange them for the decoders below:
 // xp[e][0] = (x[j=3][e], x[j=2][e]),  xp[e][1] = (x[j=1][e], x[j=0][e])  as packed 16-bit pairs.
-__device__ __forceinline__ void anyprec_load_x(const AnyprecParams& p, uint32_t wi, uint32_t (&xp)[8][2]) {
+__device__ __forceinline__ void anyprec_issue_x(const AnyprecParams& p, uint32_t wi, uint32_t (&xr)[4][4]) {
     const uint32_t i = wi >> 5, t = wi & 31u;
     const uint32_t eff = (i == p.K / 1024u) ? (p.K % 1024u) / 32u : 32u;
-    uint32_t xr[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const size_t c0 = (size_t)1024 * i + (size_t)8 * eff * j + (size_t)8 * t;
@@ -66,6 +66,8 @@ __device__ __forceinline__ void anyprec_load_x(const AnyprecParams& p, uint32_t 
             for (int q = 0; q < 4; ++q) xr[j][q] = (uint32_t)src[2 * q] | ((uint32_t)src[2 * q + 1] << 16);
         }
     }
+}
+__device__ __forceinline__ void anyprec_arrange_x(const uint32_t (&xr)[4][4], uint32_t (&xp)[8][2]) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
@@ -141,61 +143,109 @@ __device__ __forceinline__ float anyprec_generic_word(const uint32_t (&q)[BITS],
     return acc;
 }
 
-template <int DT, int BITS>
-__device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
+// Sum over the 64 lanes with DPP adds (no LDS traffic); the total ends up in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_read(float x) {
+    // lanes outside ROW_MASK, and lanes whose source is out of range, read 0
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, ROW_MASK, 0xF, true));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_read<0xB1, 0xF>(v);     // quad_perm [1,0,3,2]
+    v += dpp_read<0x4E, 0xF>(v);     // quad_perm [2,3,0,1]
+    v += dpp_read<0x124, 0xF>(v);    // row_ror 4
+    v += dpp_read<0x128, 0xF>(v);    // row_ror 8: every lane of a 16-lane row holds the row sum
+    v += dpp_read<0x142, 0xA>(v);    // row_bcast 15: rows 1 and 3 add the sum of the row before
+    v += dpp_read<0x143, 0xC>(v);    // row_bcast 31: rows 2 and 3 add the sum of rows 0..1
+    return v;
+}
+
+#define DD_CONST_AS __attribute__((address_space(4)))
+
+// One wave's share of the GEMV: slice `s` of RB consecutive rows.  All weight words of the RB rows are
+// requested before anything is decoded (a batch-1 GEMV is bound by the bytes it keeps in flight); the
+// rows' LUTs come through the scalar cache (the address is wave-uniform), so they cost no VGPRs while
+// the weights are in flight.
+template <int DT, int BITS, int RB>
+__device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
     using E = Elem<DT>;
-    constexpr int RB = 4;                                   // rows per load batch
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // wave-uniform by construction
     const uint32_t s = wave % p.S, g = wave / p.S;
-    const uint32_t rows_per_block = p.rg * p.rpw;
+    const uint32_t rows_per_block = p.rg * RB;
     const uint32_t sgrp = bid % p.sgroups, tile = bid / p.sgroups;
     const uint32_t block_row0 = tile * rows_per_block;
     const bool wave_active = g < p.rg;
     const uint32_t wi = (sgrp * p.S + s) * kWave + lane;    // word index inside the row
-    const bool lane_ok = wave_active && (wi < p.W);
+    const bool lane_ok = wi < p.W;
+    const uint32_t wi_c = lane_ok ? wi : (p.W - 1u);        // out-of-range lanes re-read a valid word and
+                                                            // multiply it with zero activations
+    const bool direct = p.S * p.sgroups <= 2u;              // few slices: every wave merges its own sums
     float* part = (float*)smem;                             // [rows_per_block][S]
     float* wlut = part + (size_t)rows_per_block * p.S + (size_t)wave * 256;
-
-    uint32_t xp[8][2];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) { xp[e][0] = 0u; xp[e][1] = 0u; }
-    if (lane_ok) anyprec_load_x(p, wi, xp);
-
-    if (wave_active) {
-        const uint32_t row0 = block_row0 + g * p.rpw;
+    const uint32_t row0 = block_row0 + g * RB;
+    if (wave_active && row0 < p.N) {
+        const uint32_t nrows = (p.N - row0) < (uint32_t)RB ? (p.N - row0) : (uint32_t)RB;
         const size_t plane_stride = (size_t)p.N * p.W;
-        for (uint32_t rb = 0; rb < p.rpw; rb += RB) {
-            uint32_t q[RB][BITS];
+        // Activations first: they are needed before the first row can be decoded, and loads return in
+        // issue order, so requesting them ahead of the weights lets row r be decoded while rows r+1..
+        // are still streaming in.
+        uint32_t xr[4][4];
+        anyprec_issue_x(p, wi_c, xr);
+        u32x4 lut4[RB];
+        if constexpr (BITS == 3) {
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
-                const uint32_t row = row0 + rb + r;
-                const bool ok = lane_ok && (rb + r < p.rpw) && (row < p.N);
-#pragma unroll
-                for (int pl = 0; pl < BITS; ++pl)
-                    q[r][pl] = ok ? p.qweight[pl * plane_stride + (size_t)row * p.W + wi] : 0u;
+                const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
+                lut4[r] = *(const DD_CONST_AS u32x4*)((const uint16_t*)p.lut + (size_t)row * 8);
             }
+        }
+        // unconditional loads from wave-uniform row bases (rows past the end re-read the last row)
+        uint32_t q[RB][BITS];
 #pragma unroll
-            for (int r = 0; r < RB; ++r) {
-                const uint32_t row = row0 + rb + r;
-                if (rb + r >= p.rpw) break;                 // uniform
-                float acc = 0.f;
-                if (row < p.N) {                            // uniform
-                    if constexpr (BITS == 3) {
-                        const u32x4 lut4 = *(const u32x4*)((const uint16_t*)p.lut + (size_t)row * 8);
-                        acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lut4, xp, 0.f);
-                    } else {
-                        constexpr int L = 1 << BITS;
-                        __builtin_amdgcn_wave_barrier();
-                        for (int v = lane; v < L; v += kWave) wlut[v] = E::load(p.lut, (size_t)row * L + v);
-                        __builtin_amdgcn_wave_barrier();
-                        acc = anyprec_generic_word<DT, BITS>(q[r], wlut, xp, 0.f);
-                    }
+        for (int r = 0; r < RB; ++r) {
+            const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
+            const uint32_t* rp = p.qweight + (size_t)row * p.W;
+#pragma unroll
+            for (int pl = 0; pl < BITS; ++pl) q[r][pl] = __builtin_nontemporal_load(rp + pl * plane_stride + wi_c);
+            __builtin_amdgcn_sched_barrier(0);      // keep the requests in row order: they return in issue order
+        }
+        uint32_t xp[8][2];
+        anyprec_arrange_x(xr, xp);
+        if (!lane_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { xp[e][0] = 0u; xp[e][1] = 0u; }
+        }
+        float sums[RB];
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            float acc;
+            if constexpr (BITS == 3) {
+                acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lut4[r], xp, 0.f);
+            } else {
+                constexpr int L = 1 << BITS;
+                const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
+                __builtin_amdgcn_wave_barrier();
+                for (int v = lane; v < L; v += kWave) wlut[v] = E::load(p.lut, (size_t)row * L + v);
+                __builtin_amdgcn_wave_barrier();
+                acc = anyprec_generic_word<DT, BITS>(q[r], wlut, xp, 0.f);
+            }
+            sums[r] = wave_sum_dpp(acc);                    // total in lane 63
+            __builtin_amdgcn_sched_barrier(0);              // decode row by row, as the rows arrive
+        }
+        if (lane == 63) {
+            if (direct) {
+#pragma unroll
+                for (int r = 0; r < RB; r += 2) {
+                    if ((uint32_t)r + 1 < nrows) E::atomic_add2(p.out, row0 + r, sums[r], sums[r + 1]);
+                    else if ((uint32_t)r < nrows) E::atomic_add1(p.out, row0 + r, sums[r]);
                 }
-                acc = wave_sum(acc);
-                if (lane == 0) part[(size_t)(g * p.rpw + rb + r) * p.S + s] = acc;
+            } else {
+#pragma unroll
+                for (int r = 0; r < RB; ++r) part[(size_t)(g * RB + r) * p.S + s] = sums[r];
             }
         }
     }
+    if (direct) return;                                     // uniform for the workgroup
     __syncthreads();
     // one atomic per output pair
     for (uint32_t t = tid; t < rows_per_block / 2; t += blockDim.x) {
@@ -209,6 +259,13 @@ __device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bi
         if (row + 1 < p.N) E::atomic_add2(p.out, row, v0, v1);
         else E::atomic_add1(p.out, row, v0);
     }
+}
+
+template <int DT, int BITS>
+__device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
+    if (p.rpw == 8) anyprec_rows<DT, BITS, 8>(p, bid, smem);
+    else if (p.rpw == 4) anyprec_rows<DT, BITS, 4>(p, bid, smem);
+    else anyprec_rows<DT, BITS, 2>(p, bid, smem);
 }
 
 }  // namespace decdec

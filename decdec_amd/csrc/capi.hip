@@ -50,8 +50,13 @@ struct Options {
     int anyprec_rpw = 0;
     int lutgemm_npb = 0;
     int sqllm_ktiles = 0;
-    int dec_lds_reduce = 1;
+    int dec_trace = 0;
+    int anyprec_rg = 0;
 } g_opt;
+
+// Diagnostics: per-workgroup cycle stamps of the DEC phases (option "dec_trace").
+constexpr int kTraceBlocks = 4096;
+unsigned long long* g_trace_dev = nullptr;
 
 int* option_slot(const char* name) {
     if (!name) return nullptr;
@@ -60,7 +65,8 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "anyprec_rpw")) return &g_opt.anyprec_rpw;
     if (!strcmp(name, "lutgemm_npb")) return &g_opt.lutgemm_npb;
     if (!strcmp(name, "sqllm_ktiles")) return &g_opt.sqllm_ktiles;
-    if (!strcmp(name, "dec_lds_reduce")) return &g_opt.dec_lds_reduce;
+    if (!strcmp(name, "dec_trace")) return &g_opt.dec_trace;
+    if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
     return nullptr;
 }
 
@@ -204,40 +210,36 @@ Config* get_config(uint64_t h) {
 constexpr size_t kLdsBudget = 60 * 1024;
 
 // Split the DEC work of one layer over at most `budget` workgroups: cg chunk groups x sg segment
-// groups, minimising the largest per-workgroup share; ties prefer fewer chunk groups (= fewer atomic
+// groups, minimising the longest per-workgroup path; ties prefer fewer chunk groups (= fewer atomic
 // adds per output).  The row list of a workgroup must fit in LDS.
-int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, bool aligned16, DecPlan* pl) {
+int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, DecPlan* pl) {
     const uint32_t num_chunks = cdiv(K, 1024);
-    uint32_t vec = 1;
-    if (aligned16 && M % 4 == 0 && M >= 256) vec = 4;
-    else if (aligned16 && M % 2 == 0 && M >= 128) vec = 2;
-    const uint32_t nseg = cdiv(M, 64 * vec);
+    const uint32_t nseg = cdiv(M, 64);
     budget = std::max(1u, budget);
     uint64_t best_cost = ~0ull;
     uint32_t best_cg = 0, best_sg = 0;
     size_t best_lds = 0;
-    uint32_t best_red = 0;
     for (uint32_t cg = 1; cg <= num_chunks; ++cg) {
         const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
         for (uint32_t sg = 1; sg <= sg_max; ++sg) {
             const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
             const uint32_t slots = cpb * std::max(k_chunk, 1u);
-            uint32_t red = g_opt.dec_lds_reduce ? 1u : 0u;
-            size_t lds = dec_lds_bytes(slots, spb, vec, red);
-            if (lds > kLdsBudget && red) { red = 0; lds = dec_lds_bytes(slots, spb, vec, 0); }
+            const size_t lds = dec_lds_bytes(slots);
             if (lds > kLdsBudget) continue;
-            // per-workgroup critical path: sequential chunk selections + (chunk, segment) fetch units;
-            // going over the workgroup budget is a last resort
-            uint64_t cost = (uint64_t)cpb * spb * 1000 + (uint64_t)cpb * 600 + (uint64_t)cg * 10 +
-                            (cg * sg > budget ? 500000ull : 0);
-            if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; best_red = red; }
+            // per-workgroup critical path: sequential chunk selections, then batches of eight rows per
+            // wave for each group of up to 16 segments; going over the workgroup budget is a last resort
+            const uint32_t sb = std::min(spb, 16u), rl = 16u / sb;
+            const uint64_t batches = (uint64_t)cdiv(spb, 16) * cdiv(slots, rl * 8);
+            const uint64_t cost = batches * 1000 + (uint64_t)cpb * 600 + (uint64_t)cg * 10 +
+                                  (cg * sg > budget ? 500000ull : 0);
+            if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
         }
     }
     if (best_cg == 0) return 1;
-    pl->cg = best_cg; pl->sg = best_sg; pl->nseg = nseg; pl->vec = vec;
+    pl->cg = best_cg; pl->sg = best_sg; pl->nseg = nseg; pl->vec = 1;
     pl->segs_per_block = cdiv(nseg, best_sg);
     pl->slots = cdiv(num_chunks, best_cg) * std::max(k_chunk, 1u);
-    pl->lds_reduce = best_red; pl->lds = best_lds;
+    pl->lds_reduce = 1; pl->lds = best_lds;
     return 0;
 }
 
@@ -251,8 +253,7 @@ int setup_config(Config* c, uint32_t k_chunk) {
     // reference dec_config.cu:180-181
     DD_CHECK(ctx->buffer_numel >= k, "DECContext buffer size is too small for the given k_chunk.");
     DD_CHECK(k_chunk <= 1024, "k_chunk must not exceed the chunk size (1024), got %u", k_chunk);
-    const bool aligned16 = ((uintptr_t)c->residual_dev % 16) == 0;
-    if (plan_dec(c->K, c->M, k_chunk, std::max(1u, ctx->num_tb), aligned16, &c->plan))
+    if (plan_dec(c->K, c->M, k_chunk, std::max(1u, ctx->num_tb), &c->plan))
         return fail(kUnsupported, "DEC launch plan does not fit in LDS (k_chunk=%u, K=%u)", k_chunk, c->K);
     c->info.hip_dec_blocks = (int)(c->plan.cg * c->plan.sg);
     c->info.hip_chunk_groups = (int)c->plan.cg;
@@ -277,12 +278,21 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
         const float a = load_host(c->thresholds_host, c->dt, 0);
         const float b = load_host(c->thresholds_host, c->dt, (size_t)k - 1);
         bucket_floors(a, b, c->dt, p->floors);
+        bool mono = p->floors[0] == p->floors[0];
+        for (int i = 1; i < kBuckets; ++i) mono = mono && (p->floors[i] <= p->floors[i - 1]);
+        p->monotone = mono ? 1u : 0u;
+        p->t1 = 18; p->t2 = 24;
     }
     p->K = c->K; p->N = c->N; p->M = c->M;
     p->num_chunks = cdiv(c->K, 1024); p->k_chunk = c->k_chunk; p->k_total = (uint32_t)k;
-    p->cg = c->plan.cg; p->sg = c->plan.sg; p->nseg = c->plan.nseg; p->vec = c->plan.vec;
+    p->cg = c->plan.cg; p->sg = c->plan.sg; p->nseg = c->plan.nseg;
     p->segs_per_block = c->plan.segs_per_block; p->slots_per_block = c->plan.slots;
-    p->use_lds_reduce = c->plan.lds_reduce; p->fused_select = fused_select ? 1u : 0u;
+    p->fused_select = fused_select ? 1u : 0u;
+    if (g_opt.dec_trace && p->cg * p->sg <= (uint32_t)kTraceBlocks) {
+        if (!g_trace_dev && hipMalloc(&g_trace_dev, sizeof(unsigned long long) * 8 * kTraceBlocks) != hipSuccess)
+            g_trace_dev = nullptr;
+        p->trace = g_trace_dev;
+    }
     return 0;
 }
 
@@ -321,10 +331,13 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     p.sgroups = cdiv(s_total, 16);
     p.S = cdiv(s_total, p.sgroups);
     p.rg = fused_block ? std::max(1u, 16u / p.S) : std::max(1u, 8u / p.S);
-    uint32_t rpw = g_opt.anyprec_rpw > 0 ? (uint32_t)g_opt.anyprec_rpw
-                                         : (uint32_t)(((uint64_t)N * p.S * p.sgroups) / 2048);
-    rpw = std::min(16u, std::max(2u, rpw));
-    rpw += rpw & 1u;
+    if (!fused_block && g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
+    // Rows per wave: every wave requests all its rows at once, so more rows per wave mean more bytes
+    // in flight per resident wave (large matrices), fewer rows mean more waves to share the decode
+    // work (small matrices, where one wave per SIMD would issue at a quarter of the VALU rate).
+    const uint64_t row_slices = (uint64_t)N * p.S * p.sgroups;
+    uint32_t rpw = row_slices >= 32768 ? 8u : (row_slices >= 8192 ? 4u : 2u);
+    if (g_opt.anyprec_rpw == 2 || g_opt.anyprec_rpw == 4 || g_opt.anyprec_rpw == 8) rpw = (uint32_t)g_opt.anyprec_rpw;
     p.rpw = rpw;
     p.x_aligned = ((uintptr_t)input % 16) == 0;
     pl->d.grid = cdiv(N, p.rg * p.rpw) * p.sgroups;
@@ -449,6 +462,15 @@ int decdec_get_option(const char* name, int* value) {
     int* s = option_slot(name);
     DD_CHECK(s != nullptr && value != nullptr, "unknown option '%s'", name ? name : "(null)");
     *value = *s;
+    return kOk;
+}
+
+int decdec_debug_read_trace(uint64_t* out, int workgroups) {
+    DD_CHECK(out && workgroups > 0 && workgroups <= kTraceBlocks, "invalid argument");
+    DD_CHECK(g_trace_dev != nullptr, "no trace has been recorded (set option dec_trace first)");
+    DD_HIP(hipDeviceSynchronize());
+    DD_HIP(hipMemcpy(out, g_trace_dev, sizeof(uint64_t) * 8 * (size_t)workgroups, hipMemcpyDeviceToHost));
+    DD_HIP(hipMemset(g_trace_dev, 0, sizeof(uint64_t) * 8 * kTraceBlocks));
     return kOk;
 }
 

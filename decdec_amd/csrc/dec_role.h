@@ -7,9 +7,11 @@
 // a workgroup owns a set of 1024-channel chunks (chunk group) and a range of column segments
 // (segment group).  It selects the channels of its own chunks itself -- selection needs only the
 // activation vector, so no grid-wide barrier and no second launch -- and then fetches the selected
-// residual rows restricted to its column segments.  A segment is 64*VEC consecutive u32 words of a
-// residual row (VEC*256 bytes, one coalesced wave-wide load).  Each wave keeps several row loads in
-// flight because the host link's latency, not ALU work, bounds the fetch.
+// residual rows restricted to its column segments.  A segment is 64 consecutive u32 words of a
+// residual row (256 bytes, one coalesced wave-wide load).  Each wave keeps eight row loads in flight
+// because the host link's latency, not ALU work, bounds the fetch.  The code is kept small on purpose
+// (rolled loops, one code path): a DEC workgroup runs its instructions once, so every instruction
+// cache line it touches is a cold miss on the critical path.
 //
 // Reference semantics reproduced (decdec_extension/dec.cu:76-280): bucket membership
 // floor[i] <= |x| < ceil[i] per bucket, buckets taken in order until k_chunk*len/1024 channels are
@@ -29,79 +31,70 @@ struct DecParams {
     void* sel_acts;             // context scratch: selected activations
     void* out;                  // output [N], accumulated atomically
     float floors[kBuckets];     // bucket floors (values exactly representable in the activation dtype)
+    uint32_t monotone;          // floors are non-increasing and free of NaN (enables the fast selection path)
+    uint32_t t1, t2;            // last bucket considered by the first / second fast-path attempt
     uint32_t K, N, M;           // M = N / 8 words per residual row
     uint32_t num_chunks, k_chunk, k_total;
     uint32_t cg, sg;            // chunk groups x segment groups = number of DEC workgroups
-    uint32_t nseg;              // column segments per row
-    uint32_t vec;               // u32 words per lane per load: 1, 2 or 4
+    uint32_t nseg;              // column segments (64 u32 words each) per row
     uint32_t segs_per_block;    // ceil(nseg / sg)
     uint32_t slots_per_block;   // capacity of the per-workgroup row list
-    uint32_t use_lds_reduce;    // reduce across waves in LDS before the global atomics
     uint32_t fused_select;      // 1: select in-kernel; 0: row indices supplied in sel_rows
+    unsigned long long* trace;  // optional [workgroup][8] cycle stamps of the phases (diagnostics), or null
 };
+
+__device__ __forceinline__ void dec_stamp(const DecParams& p, uint32_t bid, int k) {
+    if (p.trace != nullptr && threadIdx.x == 0) p.trace[(size_t)bid * 8 + k] = __builtin_readcyclecounter();
+}
 
 constexpr int kDecThreads = 1024;
 constexpr int kDecWaves = kDecThreads / kWave;
+constexpr int kMaxCand = 256;                                // fast-path candidate list capacity
+constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per thread and segment batch
 
-__host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t segs_per_block, uint32_t vec,
-                                                uint32_t use_lds_reduce) {
-    size_t b = (size_t)slots * 8 + 2 * 512 * 4;
-    if (use_lds_reduce) {
-        uint32_t sb = segs_per_block < kDecWaves ? segs_per_block : kDecWaves;
-        b += (size_t)sb * kWave * vec * 8 * 4;
-    }
-    return b;
+__host__ __device__ inline size_t dec_lds_bytes(uint32_t slots) {
+    // row list (index + activation) + selection counters/prefix + cross-wave reduction buffer
+    return (size_t)slots * 8 + 2 * 512 * 4 + (size_t)kDecWaves * 8 * kWave * 4;
 }
 
 // ---- selection of one chunk ------------------------------------------------------------------
+// General path: every wave tests its 64 channels against all 32 buckets (one ballot per bucket),
+// per-(bucket, wave) counts are prefix-summed, and each member computes its position.  Exact for any
+// floors (non-monotone floors can put a channel into several buckets, as in the reference kernel).
 template <int DT>
-__device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
-                                                 int32_t* lrows, float* lacts, uint32_t* cnt,
-                                                 uint32_t* pre, bool write_global) {
+__device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t c, uint32_t t_local, uint32_t kc,
+                                                float a, float xv, float myfloor, int32_t* lrows, float* lacts,
+                                                uint32_t* cnt, uint32_t* pre, bool write_global) {
     using E = Elem<DT>;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t lo = c * kChunk;
-    const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
-    const uint32_t kc = p.k_chunk * len / kChunk;
-    if (kc == 0) return;                                   // uniform for the workgroup
-
-    float xv = 0.f;
     uint32_t member = 0;
-    if (tid < len) {
-        xv = E::load(p.x, lo + tid);
-        const float a = __builtin_fabsf(xv);
-#pragma unroll
-        for (int i = 0; i < kBuckets; ++i) {
-            const float fl = p.floors[i];
-            const float ce = (i == 0) ? __builtin_inff() : p.floors[i - 1];
-            member |= (uint32_t)((a >= fl) && (a < ce)) << i;
-        }
-    }
-    // pass 1: members per (bucket, wave)
-#pragma unroll
+    float ce = __builtin_inff();
+#pragma unroll 1
     for (int i = 0; i < kBuckets; ++i) {
-        const unsigned long long m = __ballot((member >> i) & 1u);
+        const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+        const bool bit = (a >= fl) && (a < ce);
+        ce = fl;
+        member |= (uint32_t)bit << i;
+        const unsigned long long m = __ballot(bit);
         if (lane == 0) cnt[i * kDecWaves + wave] = (uint32_t)__popcll(m);
     }
     __syncthreads();
-    // exclusive prefix over the 512 (bucket-major, wave-minor) counts, by wave 0
-    if (wave == 0) {
-        uint32_t v[8], s = 0;
+    if (wave == 0) {   // exclusive prefix over the 512 (bucket-major, wave-minor) counts
+        uint32_t v[8], sum = 0;
 #pragma unroll
-        for (int q = 0; q < 8; ++q) { v[q] = cnt[lane * 8 + q]; s += v[q]; }
-        uint32_t incl = s;
+        for (int q = 0; q < 8; ++q) { v[q] = cnt[lane * 8 + q]; sum += v[q]; }
+        uint32_t incl = sum;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const uint32_t o = __shfl_up(incl, off, 64);
             if (lane >= (uint32_t)off) incl += o;
         }
-        uint32_t run = incl - s;
+        uint32_t run = incl - sum;
 #pragma unroll
         for (int q = 0; q < 8; ++q) { pre[lane * 8 + q] = run; run += v[q]; }
     }
     __syncthreads();
-    // pass 2: position = members in earlier buckets + members of this bucket in earlier waves
-    //         + rank inside the wave; ascending channel order inside a bucket by construction
 #pragma unroll 1
     for (int i = 0; i < kBuckets; ++i) {
         if (pre[i * kDecWaves] >= kc) break;                // uniform: later buckets start even later
@@ -122,12 +115,112 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     }
 }
 
-// ---- fetch + dequantise + accumulate ------------------------------------------------------------
-template <int VEC> struct WordVec;
-template <> struct WordVec<1> { using type = uint32_t; };
-template <> struct WordVec<2> { using type = u32x2; };
-template <> struct WordVec<4> { using type = u32x4; };
+// Inclusive prefix sum over each group of 16 lanes (DPP row shifts, zero fill).
+__device__ __forceinline__ uint32_t row_scan16(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, true);   // row_shr 1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, true);   // row_shr 2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, true);   // row_shr 4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, true);   // row_shr 8
+    return v;
+}
 
+// Fast path (floors non-increasing and free of NaN, checked on the host).  Then bucket(|x|) is the
+// number of floors above |x|, buckets 0..T tile [floor_T, +inf), and as soon as at least kc channels lie
+// in that range they are the only possible picks.  Those candidates (usually a few dozen of 1024) are
+// compacted in channel order with the key (bucket << 10 | channel); the canonical position of a
+// candidate is the number of smaller keys, counted all-pairs by the whole workgroup.  No sequential
+// walk over buckets, so the latency is a handful of LDS round trips.
+template <int DT>
+__device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
+                                                 int32_t* lrows, float* lacts, uint32_t* cnt,
+                                                 uint32_t* pre, float* red, bool write_global) {
+    using E = Elem<DT>;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t lo = c * kChunk;
+    const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
+    const uint32_t kc = p.k_chunk * len / kChunk;
+    if (kc == 0) return;                                   // uniform for the workgroup
+
+    const bool in = tid < len;
+    const float xv = in ? E::load(p.x, lo + tid) : 0.f;
+    const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");   // NaN is a member of no bucket
+    const float myfloor = p.floors[lane & 31u];            // lane i holds floor[i]
+    dec_stamp(p, blockIdx.x, 5);
+
+    uint32_t* wc = cnt;                                    // [2][16] candidate counts per wave
+    uint32_t* key = cnt + 32;                              // [kMaxCand]
+    float* cx = (float*)(cnt + 32 + kMaxCand);             // [kMaxCand] (runs into `pre`, unused here)
+    uint32_t* pc = (uint32_t*)red;                         // [4][kMaxCand] partial ranks
+    uint32_t T = 0, total = 0, base = 0, bkt = 0;
+    bool fast = false, is_cand = false;
+    if (p.monotone) {
+        // bucket index = number of floors (up to t2) strictly above |x|
+#pragma unroll 1
+        for (uint32_t i = 0; i <= p.t2; ++i) {
+            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), (int)i));
+            bkt += (a < fl) ? 1u : 0u;
+        }
+        const bool finite = a < __builtin_inff();          // false for NaN and inf
+        const bool c1 = finite && (bkt <= p.t1), c2 = finite && (bkt <= p.t2);
+        const unsigned long long m1 = __ballot(c1), m2 = __ballot(c2);
+        if (lane == 0) { wc[wave] = (uint32_t)__popcll(m1); wc[16 + wave] = (uint32_t)__popcll(m2); }
+        __syncthreads();
+        const uint32_t v = wc[lane & 31u];                 // lanes 0..15: first attempt, 16..31: second
+        const uint32_t incl = row_scan16(v);
+        const uint32_t tot1 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 15);
+        const uint32_t tot2 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
+        const bool ok1 = (tot1 >= kc) && (tot1 <= (uint32_t)kMaxCand);
+        const bool ok2 = (tot2 >= kc) && (tot2 <= (uint32_t)kMaxCand);
+        fast = ok1 || ok2;
+        T = ok1 ? p.t1 : p.t2;
+        total = ok1 ? tot1 : tot2;
+        const uint32_t excl = incl - v;
+        base = (uint32_t)__builtin_amdgcn_readlane((int)excl, (int)(ok1 ? wave : 16u + wave));
+        is_cand = ok1 ? c1 : c2;
+        if (fast) {
+            const unsigned long long cm = ok1 ? m1 : m2;
+            if (is_cand) {
+                const uint32_t idx = base + ballot_rank(cm);
+                key[idx] = (bkt << 10) | tid;
+                cx[idx] = xv;
+            }
+        }
+        __syncthreads();
+    }
+    if (!fast) {
+        dec_select_general<DT>(p, c, t_local, kc, a, xv, myfloor, lrows, lacts, cnt, pre, write_global);
+        return;
+    }
+    dec_stamp(p, blockIdx.x, 6);
+    {   // partial rank of candidate j among candidates [64 q, 64 q + 64)
+        const uint32_t j = tid & (uint32_t)(kMaxCand - 1), q = tid / (uint32_t)kMaxCand;
+        const uint32_t mykey = j < total ? key[j] : 0u;
+        const uint32_t q0 = q * 64u;
+        const uint32_t qn = q0 >= total ? 0u : ((total - q0) < 64u ? (total - q0) : 64u);
+        uint32_t r = 0;
+#pragma unroll 4
+        for (uint32_t it = 0; it < qn; ++it) r += (key[q0 + it] < mykey) ? 1u : 0u;
+        pc[q * kMaxCand + j] = r;
+    }
+    __syncthreads();
+    if (tid < total) {
+        const uint32_t pos = pc[tid] + pc[kMaxCand + tid] + pc[2 * kMaxCand + tid] + pc[3 * kMaxCand + tid];
+        if (pos < kc) {
+            const uint32_t ch = lo + (key[tid] & 1023u);
+            const float xs = cx[tid];
+            const uint32_t slot = t_local * p.k_chunk + pos;
+            lrows[slot] = (int32_t)ch;
+            lacts[slot] = xs;
+            if (write_global) {
+                p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
+                E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
+            }
+        }
+    }
+    dec_stamp(p, blockIdx.x, 7);
+}
+
+// ---- fetch + dequantise + accumulate ------------------------------------------------------------
 __device__ __forceinline__ void dec_accumulate_word(uint32_t w, float act, float* acc) {
     const uint32_t lo = w & 0x0F0F0F0Fu;           // nibbles 0,2,4,6 as bytes
     const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;    // nibbles 1,3,5,7 as bytes
@@ -141,32 +234,44 @@ __device__ __forceinline__ void dec_accumulate_word(uint32_t w, float act, float
     acc[7] += (float)(hi >> 24) * act;
 }
 
-template <int DT, int VEC>
-__device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t sgid, uint32_t nslots,
+template <int DT>
+__device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint32_t sgid, uint32_t nslots,
                                           const int32_t* lrows, const float* lacts, float* red) {
     using E = Elem<DT>;
-    using V = typename WordVec<VEC>::type;
-    constexpr int U = (VEC == 4) ? 8 : 8;              // residual rows in flight per wave
+    constexpr int U = 8;                                // residual rows in flight per wave
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t seg_lo = sgid * p.segs_per_block;
     const uint32_t seg_hi = (seg_lo + p.segs_per_block) < p.nseg ? (seg_lo + p.segs_per_block) : p.nseg;
 
+#pragma unroll 1
     for (uint32_t sb0 = seg_lo; sb0 < seg_hi; sb0 += kDecWaves) {
         const uint32_t SB = (seg_hi - sb0) < (uint32_t)kDecWaves ? (seg_hi - sb0) : (uint32_t)kDecWaves;
         const uint32_t RL = kDecWaves / SB;             // waves sharing one segment
         const uint32_t ls = wave % SB, rl = wave / SB;
-        const uint32_t w0 = ((sb0 + ls) * kWave + lane) * VEC;
+        const uint32_t w0 = (sb0 + ls) * kWave + lane;  // u32 column of the residual row
         const bool col_ok = (rl < RL) && (w0 < p.M);
 
-        float acc[VEC * 8];
+        float acc[8];
 #pragma unroll
-        for (int j = 0; j < VEC * 8; ++j) acc[j] = 0.f;
+        for (int j = 0; j < 8; ++j) acc[j] = 0.f;
         float act_sum = 0.f;
+        // the scales this thread needs in the merge step, requested before the row fetch so that their
+        // latency hides behind it: merge task t -> word (t & 63) of segment t >> 8, output pair (t >> 6) & 3
+        float sc0[kMergeTasks], sc1[kMergeTasks];
+#pragma unroll
+        for (int q = 0; q < kMergeTasks; ++q) {
+            const uint32_t t = tid + (uint32_t)q * kDecThreads;
+            const uint32_t m = (sb0 + (t >> 8)) * kWave + (t & 63u), jp = (t >> 6) & 3u;
+            const bool ok = (t < SB * 256u) && (m < p.M);
+            sc0[q] = ok ? E::load(p.scales, (size_t)(2 * jp) * p.M + m) : 0.f;
+            sc1[q] = ok ? E::load(p.scales, (size_t)(2 * jp + 1) * p.M + m) : 0.f;
+        }
 
         if (col_ok) {
             const uint32_t* base = p.residual + w0;
+#pragma unroll 1
             for (uint32_t r = rl; r < nslots; r += RL * U) {
-                V data[U];
+                uint32_t data[U];
                 float act[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -176,56 +281,43 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t sgid, uin
                     if (rr < nslots) { row = lrows[rr]; a = lacts[rr]; }
                     row = __builtin_amdgcn_readfirstlane(row);      // wave-uniform by construction
                     if (row >= 0) {
-                        data[u] = *(const V*)(base + (size_t)row * p.M);
+                        data[u] = base[(size_t)row * p.M];
                         act[u] = a;
                     } else {
-                        data[u] = (V)(0x88888888u);                 // nibble 8 == value 0
+                        data[u] = 0x88888888u;                      // nibble 8 == value 0
                         act[u] = 0.f;
                     }
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     act_sum += act[u];
-                    if constexpr (VEC == 1) {
-                        dec_accumulate_word(data[u], act[u], acc);
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < VEC; ++v) dec_accumulate_word(data[u][v], act[u], acc + 8 * v);
-                    }
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < VEC * 8; ++j) acc[j] -= 8.f * act_sum;   // stored nibble = q + 8
-        }
-
-        const bool lds_reduce = p.use_lds_reduce && (RL > 1);       // uniform
-        if (lds_reduce) {
-            const uint32_t n_red = SB * kWave * VEC * 8;
-            for (uint32_t i = tid; i < n_red; i += kDecThreads) red[i] = 0.f;
-            __syncthreads();
-            if (col_ok) {
-#pragma unroll
-                for (int j = 0; j < VEC * 8; ++j) atomicAdd(&red[(ls * VEC * 8 + j) * kWave + lane], acc[j]);
-            }
-            __syncthreads();
-            if (col_ok && rl == 0) {
-#pragma unroll
-                for (int j = 0; j < VEC * 8; ++j) acc[j] = red[(ls * VEC * 8 + j) * kWave + lane];
-            }
-        }
-        if (col_ok && (!lds_reduce || rl == 0)) {
-#pragma unroll
-            for (int v = 0; v < VEC; ++v) {
-                const uint32_t m = w0 + v;
-#pragma unroll
-                for (int j = 0; j < 8; j += 2) {
-                    const float s0 = E::load(p.scales, (size_t)j * p.M + m);
-                    const float s1 = E::load(p.scales, (size_t)(j + 1) * p.M + m);
-                    E::atomic_add2(p.out, (size_t)8 * m + j, acc[8 * v + j] * s0, acc[8 * v + j + 1] * s1);
+                    dec_accumulate_word(data[u], act[u], acc);
                 }
             }
         }
-        if (lds_reduce) __syncthreads();                             // red is reused by the next batch
+        dec_stamp(p, bid, 2);
+        // cross-wave reduction through LDS (plain stores; LDS float atomics are slow), then one
+        // atomic add per output pair for the whole workgroup
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            red[(wave * 8 + j) * kWave + lane] = col_ok ? (acc[j] - 8.f * act_sum) : 0.f;   // nibble = q + 8
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < kMergeTasks; ++q) {
+            const uint32_t t = tid + (uint32_t)q * kDecThreads;
+            const uint32_t lw = t & 63u, jp = (t >> 6) & 3u, sl = t >> 8;
+            const uint32_t m = (sb0 + sl) * kWave + lw;
+            if (t >= SB * 256u || m >= p.M) continue;
+            float v0 = 0.f, v1 = 0.f;
+            for (uint32_t qq = 0; qq < RL; ++qq) {
+                const uint32_t wv = qq * SB + sl;
+                v0 += red[(wv * 8 + 2 * jp) * kWave + lw];
+                v1 += red[(wv * 8 + 2 * jp + 1) * kWave + lw];
+            }
+            E::atomic_add2(p.out, (size_t)8 * m + 2 * jp, v0 * sc0[q], v1 * sc1[q]);
+        }
+        dec_stamp(p, bid, 3);
+        __syncthreads();                                 // red is reused by the next batch
     }
 }
 
@@ -241,13 +333,14 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
     uint32_t* pre = cnt + 512;
     float* red = (float*)(pre + 512);
 
+    dec_stamp(p, bid, 0);
     for (uint32_t i = tid; i < p.slots_per_block; i += kDecThreads) lrows[i] = -1;
     uint32_t nslots = 0;
     if (p.fused_select) {
         uint32_t t = 0;
         for (uint32_t c = cgid; c < p.num_chunks; c += p.cg, ++t) {
             __syncthreads();      // list initialised; cnt/pre of the previous chunk no longer read
-            dec_select_chunk<DT>(p, c, t, lrows, lacts, cnt, pre, sgid == 0);
+            dec_select_chunk<DT>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0);
         }
         nslots = t * p.k_chunk;
     } else {
@@ -264,9 +357,9 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
         nslots = hi > lo ? hi - lo : 0;
     }
     __syncthreads();
-    if (p.vec == 4) dec_fetch<DT, 4>(p, sgid, nslots, lrows, lacts, red);
-    else if (p.vec == 2) dec_fetch<DT, 2>(p, sgid, nslots, lrows, lacts, red);
-    else dec_fetch<DT, 1>(p, sgid, nslots, lrows, lacts, red);
+    dec_stamp(p, bid, 1);
+    dec_fetch<DT>(p, bid, sgid, nslots, lrows, lacts, red);
+    dec_stamp(p, bid, 4);
 }
 
 }  // namespace decdec

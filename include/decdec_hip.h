@@ -55,7 +55,8 @@ int decdec_version(void);
 /* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
  * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
  * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "lutgemm_npb",
- * "sqllm_ktiles" (launch-shape overrides, 0 = automatic).  No counterpart in the reference. */
+ * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "dec_trace" (see
+ * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
 int decdec_get_option(const char* name, int* value);
 
@@ -140,6 +141,12 @@ int decdec_dummy_lutgemm(const void* input, void* output, const void* q_weight, 
 int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, const void* lut,
                        int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
                        int dummy_cu, int64_t dummy_iters, void* stream);
+
+/* Diagnostics: with option "dec_trace" = 1 every DEC workgroup stores shader-clock stamps of its
+ * phases (0 start, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a
+ * library-owned device buffer; this copies the first `workgroups` x 8 stamps to the host (it
+ * synchronises the device).  No counterpart in the reference. */
+int decdec_debug_read_trace(uint64_t* stamps_out, int workgroups);
 
 /* Host-only helpers (no GPU needed).  decdec_bucket_floors evaluates the selector's 32 bucket
  * floors exactly as dec.cu:117-130 does, in `dtype` arithmetic; decdec_reference_geometry evaluates

@@ -33,8 +33,17 @@ def make_dec_layer(K, N, seed, dtype=torch.float16, random_residual=False):
             "cheat": cheat.contiguous(), "scales": scales.to(dtype).contiguous(), "x": x, "th": th}
 
 
-def rel_err(got: np.ndarray, want: np.ndarray):
-    """(max relative error with a floor of 1e-2*max|want| in the denominator, mean abs error)."""
+REL_FLOOR = 0.1
+
+
+def rel_err(got: np.ndarray, want: np.ndarray, floor: float = REL_FLOOR):
+    """(max relative error, mean abs error) of ``got`` against the float64 oracle ``want``.
+
+    The denominator is max(|want_i|, floor * max|want|).  Outputs are fp16 sums of terms that cancel,
+    so an output near zero carries the absolute rounding error of partial sums as large as max|want|;
+    with a 1 % floor the reference's own fp16 arithmetic (oracle.dec_apply_reference_rounding) scores
+    4.4e-2 on the 4096x4096, k_chunk=32 case, above the 1e-2 tolerance, and 5.5e-3 with the 10 %
+    floor used here (tests/test_oracle.py::test_reference_rounding_error_budget)."""
     got = got.astype(np.float64); want = want.astype(np.float64)
-    denom = np.maximum(np.abs(want), 1e-2 * np.max(np.abs(want)) + 1e-30)
+    denom = np.maximum(np.abs(want), floor * np.max(np.abs(want)) + 1e-30)
     return float(np.max(np.abs(got - want) / denom)), float(np.mean(np.abs(got - want)))
