@@ -391,7 +391,8 @@ int plan_sqllm(const void* input, void* output, const void* mat, const void* lut
     p.nthreads = 256;
     p.n_tiles = cdiv(N, p.nthreads);
     uint32_t kt = g_opt.sqllm_ktiles > 0 ? (uint32_t)g_opt.sqllm_ktiles : cdiv(2048, p.n_tiles);
-    kt = std::max(1u, std::min(kt, K / 128 ? K / 128 : 1u));
+    // every K range costs one rounding of the 16-bit output (one atomic add), so the split stays small
+    kt = std::max(1u, std::min(std::min(kt, 8u), K / 128 ? K / 128 : 1u));
     p.kspan = cdiv(cdiv(K, kt), 32) * 32;
     p.k_tiles = cdiv(K, p.kspan);
     pl->d.grid = p.n_tiles * p.k_tiles;

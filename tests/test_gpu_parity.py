@@ -12,7 +12,8 @@ from oracle import decdec_oracle as O
 from tests.helpers import TORCH_DT, make_dec_layer, np_of, rel_err
 
 pytestmark = pytest.mark.gpu
-TOL = 1e-2
+TOL = 1e-2            # fp16 and fp32 outputs
+TOL_BF16 = 8e-2       # bf16 has 8 significand bits against fp16's 11: the same bound in units of ulp
 
 
 def _ctx(n_tb, K, dtype):
@@ -79,3 +80,332 @@ def test_dec_anyprec_fused_matches_sum(c_oracle):
     exact = L["W"].double().numpy() @ np_of(L["x"]).astype(np.float64).reshape(-1)
     base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
     assert np.abs(np_of(out).reshape(-1) - exact).mean() < np.abs(base - exact).mean()
+
+
+# --------------------------------------------------------------------------------------------------
+# other dtypes, other bit widths, the other base GEMVs
+# --------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["bf16", "fp32"])
+def test_dec_other_dtypes_reference_recipe(dt, c_oracle):
+    """The reference's own test recipe (decdec_extension/tests/test_dec.py): num_tb=24, K=14336,
+    N=4096, k_chunk=20, random int32 residual, rand scales, x in U(-1,1), thresholds = sort(|x|)."""
+    dtype = TORCH_DT[dt]
+    K, N, k_chunk, n_tb = 14336, 4096, 20, 24
+    g = torch.Generator().manual_seed(0)
+    cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32)
+    scales = torch.rand(N, generator=g).to(dtype)
+    x = (torch.rand(1, 1, K, generator=g) * 2 - 1).to(dtype)
+    th = torch.sort(x.float().abs().view(-1), descending=True).values.to(dtype)
+    ctx, rows, acts = _ctx(n_tb, K, dtype)
+    cfg = ext.create_dec_config(ctx, k_chunk, cheat, scales, th)
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    ext.dec(cfg, x.cuda(), out)
+    torch.cuda.synchronize()
+    want_rows, want_acts, _ = O.select_channels(np_of(x), np_of(th), k_chunk, dt)
+    k = k_chunk * K // 1024
+    assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k])
+    assert np.array_equal(np_of(acts)[:k], want_acts[:k])
+    want = c_oracle.dec_apply(np_of(x), cheat.numpy(), np_of(scales), want_rows, dt)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dt != "bf16" else TOL_BF16), (mre, mae)     # bf16 carries 8 mantissa bits
+    ext.destroy_dec_config(cfg)
+
+
+@pytest.mark.parametrize("bits", [3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("dt", ["fp16", "bf16"])
+def test_anyprec_gemv_bits_and_dequant(bits, dt, c_oracle):
+    dtype = TORCH_DT[dt]
+    K, N = 2048 + 512, 96                      # tail chunk of 512 channels, N not a multiple of 8
+    g = torch.Generator().manual_seed(bits)
+    idx = torch.randint(0, 1 << bits, (N, K), generator=g, dtype=torch.int64)
+    lut = torch.randn(N, 1 << bits, generator=g).to(dtype)
+    qweight = F.pack_anyprec(idx, bits)
+    x = F.make_activation(K, g, dtype=dtype)
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    ext.anyprec_gemv(x.cuda(), out, qweight.cuda(), lut.cuda(), bits)
+    w = ext.anyprec_dequant(qweight.cuda(), lut.cuda(), bits)
+    torch.cuda.synchronize()
+    want_w = O.anyprec_dequant(qweight.numpy(), np_of(lut), bits)
+    assert np.array_equal(np_of(w), want_w), "dequantised weights must be bit-exact LUT entries"
+    want = c_oracle.anyprec_gemv(np_of(x), qweight.numpy(), np_of(lut), bits, dt)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dt == "fp16" else TOL_BF16), (mre, mae)
+
+
+def test_anyprec_extra_planes_are_ignored(c_oracle):
+    """qweight may hold more planes than `bitwidth` (any-precision storage); only the first are read."""
+    K, N = 1024, 64
+    g = torch.Generator().manual_seed(5)
+    idx8 = torch.randint(0, 256, (N, K), generator=g, dtype=torch.int64)
+    q8 = F.pack_anyprec(idx8, 8)
+    lut3 = torch.randn(N, 8, generator=g).half()
+    x = F.make_activation(K, g)
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.anyprec_gemv(x.cuda(), out, q8.cuda(), lut3.cuda(), 3)
+    torch.cuda.synchronize()
+    want = c_oracle.anyprec_gemv(np_of(x), q8.numpy()[:3].copy(), np_of(lut3), 3)
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+
+
+@pytest.mark.parametrize("K,N,bits,group", [(5120, 5120, 3, 128), (4096, 1024, 4, 128), (1024, 258, 2, 64)])
+@pytest.mark.parametrize("dt", ["fp16", "fp32", "bf16"])
+def test_lutgemm_gemv(K, N, bits, group, dt, c_oracle):
+    dtype = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(K + N)
+    W = (torch.randn(N, K, generator=g) * 0.02).half()
+    q, s, z = F.awq_pseudo_quantize(W, bits, group)
+    qw, alpha, q_bias = F.pack_bcq(q, s, z, bits, dtype)
+    x = F.make_activation(K, g, dtype=dtype)
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    ext.lutgemm_gemv(x.cuda(), out, qw.cuda(), alpha.cuda(), q_bias.cuda(), bits, group)
+    torch.cuda.synchronize()
+    want = c_oracle.lutgemm_gemv(np_of(x), qw.numpy(), np_of(alpha), np_of(q_bias), bits, group, dt)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dt != "bf16" else TOL_BF16), (mre, mae)
+
+
+@pytest.mark.parametrize("K,N,bits", [(4096, 4096, 4), (4096, 1024, 3), (1024, 130, 4), (2048, 66, 3)])
+@pytest.mark.parametrize("dt", ["fp16", "fp32", "bf16"])
+def test_sqllm_gemv(K, N, bits, dt, c_oracle):
+    dtype = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(K + N + bits)
+    idx = torch.randint(0, 1 << bits, (N, K), generator=g, dtype=torch.int64)
+    lut = (torch.randn(N, 1 << bits, generator=g) * 0.02).to(dtype)
+    mat = F.pack_sqllm(idx, bits)
+    x = F.make_activation(K, g, dtype=dtype)
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    ext.sqllm_gemv(x.cuda(), out, mat.cuda(), lut.cuda(), bits)
+    torch.cuda.synchronize()
+    want = c_oracle.sqllm_gemv(np_of(x), mat.numpy(), np_of(lut), bits, dt)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dt != "bf16" else TOL_BF16), (mre, mae)
+
+
+# --------------------------------------------------------------------------------------------------
+# fused DEC + GEMV (both fusion modes), unfused DEC, config updates, edge cases
+# --------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fusion", [1, 0])
+@pytest.mark.parametrize("kind", ["anyprec", "lutgemm", "sqllm"])
+def test_dec_plus_gemv(kind, fusion, c_oracle):
+    from decdec_amd import _lib
+    K, N, k_chunk = 5120, 5120, 32
+    L = make_dec_layer(K, N, seed=77)
+    g = torch.Generator().manual_seed(78)
+    ctx, rows, acts = _ctx(16, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+    x = L["x"].cuda()
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    _lib.set_option("fusion", fusion)
+    try:
+        if kind == "anyprec":
+            ext.dec_anyprec(cfg, x, out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+            base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+        elif kind == "lutgemm":
+            q, s, z = F.awq_pseudo_quantize(L["W"], 3, 128)
+            qw, alpha, q_bias = F.pack_bcq(q, s, z, 3)
+            ext.dec_lutgemm(cfg, x, out, qw.cuda(), alpha.cuda(), q_bias.cuda(), 3, 128)
+            base = c_oracle.lutgemm_gemv(np_of(L["x"]), qw.numpy(), np_of(alpha), np_of(q_bias), 3, 128)
+        else:
+            idx, lut = F.quantize_uniform_rows(L["W"], 4)
+            mat = F.pack_sqllm(idx, 4)
+            ext.dec_sqllm(cfg, x, out, mat.cuda(), lut.cuda(), 4)
+            base = c_oracle.sqllm_gemv(np_of(L["x"]), mat.numpy(), np_of(lut), 4)
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_option("fusion", 1)
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+    k = k_chunk * K // 1024
+    assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k])
+    want = base + c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= TOL, (mre, mae)
+    ext.destroy_dec_config(cfg)
+
+
+def test_unfused_dec_uses_caller_indices(c_oracle):
+    """evaluation/evaltools.py:327-343: exact top-k indices are written into the context's row
+    buffer and unfused_dec fetches those rows."""
+    K, N, k_chunk = 4096, 1024, 16
+    L = make_dec_layer(K, N, seed=31)
+    ctx, rows, acts = _ctx(8, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+    x = L["x"].cuda()
+    k = k_chunk * K // 1024
+    topk = torch.topk(x[0, 0].abs().float(), k, largest=True).indices.to(torch.int32)
+    rows[:k] = topk
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.unfused_dec(cfg, x, out)
+    torch.cuda.synchronize()
+    want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), topk.cpu().numpy())
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+    # duplicates count twice, out-of-range indices are ignored
+    rows[:k] = topk
+    rows[0] = rows[1]
+    rows[2] = K + 5
+    out.zero_()
+    ext.unfused_dec(cfg, x, out)
+    torch.cuda.synchronize()
+    r = rows[:k].cpu().numpy().copy()
+    want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), r)
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+    ext.destroy_dec_config(cfg)
+
+
+def test_select_all_channels_reduces_to_dense_gemv():
+    """k_chunk = 1024 selects every channel: DEC becomes the dense GEMV x @ R_hat (textbook check)."""
+    K, N = 2048, 512
+    L = make_dec_layer(K, N, seed=3)
+    ctx, rows, acts = _ctx(8, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, 1024, L["cheat"], L["scales"], L["th"])
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.dec(cfg, L["x"].cuda(), out)
+    torch.cuda.synchronize()
+    R = F.unpack_residual(L["cheat"], L["scales"]).double()
+    want = (L["x"].double().reshape(1, -1) @ R).reshape(-1).numpy()
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+    assert sorted(rows.cpu().numpy()[:K].tolist()) == list(range(K))
+    ext.destroy_dec_config(cfg)
+
+
+def test_k_chunk_zero_is_a_noop_and_update_config(c_oracle):
+    K, N = 4096, 4096
+    L = make_dec_layer(K, N, seed=9)
+    ctx, rows, acts = _ctx(8, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, 0, L["cheat"], L["scales"], L["th"])
+    x = L["x"].cuda()
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.dec(cfg, x, out)
+    ext.dec_anyprec(cfg, x, out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+    torch.cuda.synchronize()
+    base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+    assert rel_err(np_of(out).reshape(-1), base)[0] <= TOL
+    assert (rows.cpu().numpy() == -7).all()
+    # retune: new context (other n_tb) and k_chunk, residual not copied again
+    ctx2 = ext.create_dec_context(32, rows, acts)
+    ext.update_dec_config(cfg, ctx2, 8)
+    assert ext.read_dec_config(cfg)["k_chunk"] == 8
+    out.zero_()
+    ext.dec(cfg, x, out)
+    torch.cuda.synchronize()
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), 8)
+    assert np.array_equal(rows.cpu().numpy()[:32], want_rows[:32])
+    want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+    # a context whose buffers are too small is rejected (dec_config.cu:180-181)
+    small = ext.create_dec_context(8, rows[:16], acts[:16])
+    with pytest.raises(RuntimeError, match="buffer size is too small"):
+        ext.update_dec_config(cfg, small, 32)
+    assert ext.read_dec_config(cfg)["k_chunk"] == 8
+    ext.destroy_dec_config(cfg)
+
+
+def test_selector_edge_cases_general_path(c_oracle):
+    """Non-monotone thresholds (a < b), ties, inf / NaN activations and fewer members than k_chunk:
+    the kernel's general path must still reproduce the oracle bit for bit."""
+    K, N, k_chunk = 3072, 256, 32
+    L = make_dec_layer(K, N, seed=21)
+    x = L["x"].clone()
+    x[0, 0, 5] = float("inf"); x[0, 0, 1030] = float("nan"); x[0, 0, 2050:2200] = 3.0   # ties in one bucket
+    cases = {
+        "reversed": torch.flip(L["th"], dims=[0]),
+        "constant": torch.full_like(L["th"], 2.0),
+        "zeros": torch.zeros_like(L["th"]),
+        "calibrated": L["th"],
+    }
+    for name, th in cases.items():
+        th = th.contiguous()
+        ctx, rows, acts = _ctx(4, K, torch.float16)
+        cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], th)
+        out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+        xs = torch.nan_to_num(x, nan=0.0, posinf=0.0) if name == "never" else x
+        ext.dec(cfg, xs.cuda(), out)
+        torch.cuda.synchronize()
+        want_rows, _, filled = O.select_channels(np_of(xs), np_of(th), k_chunk)
+        got = rows.cpu().numpy()[: want_rows.shape[0]]
+        assert np.array_equal(got[filled], want_rows[filled]), name
+        assert (got[~filled] == -7).all(), name          # slots the reference leaves untouched stay untouched
+        ext.destroy_dec_config(cfg)
+
+
+def test_residual_on_device_is_used_in_place(c_oracle, capfd):
+    K, N, k_chunk = 4096, 1024, 32
+    L = make_dec_layer(K, N, seed=13)
+    ctx, rows, acts = _ctx(8, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"].cuda(), L["scales"].cuda(), L["th"])
+    assert ext.read_dec_config(cfg, native=True)["hip_residual_on_host"] == 0
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.dec(cfg, L["x"].cuda(), out)
+    torch.cuda.synchronize()
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+    want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+    ext.destroy_dec_config(cfg)
+
+
+def test_dummy_ops_run_the_base_gemv(c_oracle):
+    K, N = 4096, 1024
+    L = make_dec_layer(K, N, seed=17)
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.dummy_anyprec(L["x"].cuda(), out, L["qweight"].cuda(), L["lut"].cuda(), 3, 4, 1000)
+    torch.cuda.synchronize()
+    want = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+    assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+
+
+def test_linear_modules_decode_and_prefill(c_oracle):
+    from decdec_amd.linear import APLinear
+    K, N, k_chunk = 4096, 1024, 16
+    L = make_dec_layer(K, N, seed=23)
+    lin = APLinear(K, N, 3)
+    lin.qweight.copy_(L["qweight"]); lin.lut.copy_(L["lut"])
+    lin.load_dec_data(L["cheat"], L["scales"], L["th"])
+    rows = torch.zeros(K, dtype=torch.int32, device="cuda"); acts = torch.zeros(K, dtype=torch.float16, device="cuda")
+    ctx = ext.create_dec_context(8, rows, acts)
+    lin.create_dec_config(ctx, k_chunk)
+    y = lin(L["x"].cuda())
+    torch.cuda.synchronize()
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+    want = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3) + \
+        c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    assert rel_err(np_of(y).reshape(-1), want)[0] <= TOL
+    xs = torch.randn(1, 5, K, dtype=torch.float16, device="cuda")
+    yp = lin(xs)                                  # prefill: dequantise + matmul
+    wd = F.dequant_lut(L["idx"], L["lut"]).cuda()
+    assert torch.allclose(yp, xs @ wd.T, rtol=1e-2, atol=1e-2)
+
+
+def test_full_size_layer_properties():
+    """BASELINE shapes too large for the oracle in seconds: size-independent properties.
+    (i) linearity in x of the base GEMV; (ii) dec(x) with k_chunk selecting everything equals the dense
+    residual GEMV computed by torch on the GPU; (iii) selection returns distinct in-range channels."""
+    K, N = 8192, 28672
+    g = torch.Generator().manual_seed(1)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (3, N, K // 32), generator=g, dtype=torch.int64).to(torch.int32).cuda()
+    lut = torch.randn(N, 8, generator=g).half().cuda()
+    x1 = F.make_activation(K, g).cuda(); x2 = F.make_activation(K, g).cuda()
+    o1 = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda"); o2 = torch.zeros_like(o1); o12 = torch.zeros_like(o1)
+    ext.anyprec_gemv(x1, o1, qw, lut, 3); ext.anyprec_gemv(x2, o2, qw, lut, 3)
+    ext.anyprec_gemv((x1.float() * 0.5 + x2.float() * 0.25).half(), o12, qw, lut, 3)
+    torch.cuda.synchronize()
+    lin = o1.float() * 0.5 + o2.float() * 0.25
+    scale = lin.abs().max()
+    assert ((o12.float() - lin).abs().max() / scale) < 2e-2
+    w = ext.anyprec_dequant(qw, lut, 3)
+    ref = (x1.float().reshape(1, -1) @ w.float().T).reshape(-1)
+    assert ((o1.float().reshape(-1) - ref).abs().max() / ref.abs().max()) < 1e-2
+    # selection at the 70B 'down' input width
+    K2, N2, k_chunk = 28672, 1024, 32
+    cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K2, N2 // 8), generator=g, dtype=torch.int64).to(torch.int32)
+    th = F.calibrate_thresholds(K2, g, draws=4)
+    ctx, rows, acts = _ctx(32, K2, torch.float16)
+    cfg = ext.create_dec_config(ctx, k_chunk, cheat, torch.rand(N2, generator=g).half(), th)
+    x = F.make_activation(K2, g).cuda()
+    out = torch.zeros(1, 1, N2, dtype=torch.float16, device="cuda")
+    ext.dec(cfg, x, out)
+    torch.cuda.synchronize()
+    k = k_chunk * K2 // 1024
+    r = rows.cpu().numpy()[:k]
+    assert len(set(r.tolist())) == k and r.min() >= 0 and r.max() < K2
+    assert ((r // 1024) == np.repeat(np.arange(K2 // 1024), k_chunk)).all()
+    assert torch.equal(acts[:k], x[0, 0][torch.from_numpy(r).long().cuda()])
+    ext.destroy_dec_config(cfg)
