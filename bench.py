@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the DecDEC decode linear-layer path on one MI355X.
+
+Metric (BASELINE.json): microseconds per token spent in the quantised linear layers of a
+Llama-3-8B decode step at batch 1, with DEC, plus the DEC slowdown against the base GEMVs alone.
+
+A "step" is one token: the 32 x 7 linear layers (q, k, v, o, gate, up, down; 224 layers, every one with
+its own weights in HBM -- 2.64 GB of 3-bit any-precision bitplanes, so nothing is served from a cache
+warmed by the previous step -- and its own 4-bit residual in pinned host memory, 3.3 GB) executed
+back to back through the C ABI.  The step is captured once in a HIP graph (the reference's decode
+loop runs under CUDA graphs as well, end-to-end/generate.py:115-121) and replayed; every replayed
+kernel is the library's own.  The activations, weights and residuals are synthetic (seeded).
+
+Prints ONE JSON line.  `value` = us/token with DEC (k_chunk 32, n_tb 8); `base_us_per_token` and
+`dec_slowdown_pct` sit beside it; `roofline` is the any-precision GEMV of the largest layer shape
+(4096 -> 14336) measured with HIP events on its own stream; `cpu_baseline` is the C restatement of
+the same layer path (oracle/decdec_oracle.c, OpenMP over the host cores) on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LLAMA3_8B = [("q", 4096, 4096), ("k", 4096, 1024), ("v", 4096, 1024), ("o", 4096, 4096),
+             ("gate", 4096, 14336), ("up", 4096, 14336), ("down", 14336, 4096)]
+BITS = 3
+HBM_PEAK_GBS = 8000.0
+
+
+def anyprec_bytes(K, N, bits=BITS):
+    """Algorithmic bytes of one any-precision GEMV: planes + LUT + activations + outputs."""
+    return bits * N * K // 8 + N * (1 << bits) * 2 + 2 * K + 2 * N
+
+
+def build_layer_set(torch, F, n_layers, k_chunk, seed):
+    """Synthetic Llama-3-8B linear layers in the benchmark recipe.  Quantisation is done once per shape
+    on the GPU; every layer then owns private copies of the packed weights (distinct HBM) and of the
+    residual (distinct pinned host memory)."""
+    g = torch.Generator().manual_seed(seed)
+    protos = {}
+    for name, K, N in LLAMA3_8B:
+        if (K, N) in protos:
+            continue
+        W = (torch.randn(N, K, generator=g) * 0.02).to(torch.float16).cuda()
+        idx, lut = F.quantize_uniform_rows(W, BITS)
+        qweight = F.pack_anyprec(idx, BITS)
+        resid = (W.float() - F.dequant_lut(idx, lut).float()).to(torch.float16)
+        q, s = F.quantize_residual(resid)
+        cheat, scales = F.pack_residual(q, s)
+        th = F.calibrate_thresholds(K, g, draws=32)
+        protos[(K, N)] = dict(qweight=qweight, lut=lut.contiguous(), cheat=cheat.cpu().contiguous(),
+                              scales=scales.cpu().contiguous(), th=th)
+        del W, idx, resid, q
+    torch.cuda.synchronize()
+    layers = []
+    for li in range(n_layers):
+        for name, K, N in LLAMA3_8B:
+            p = protos[(K, N)]
+            layers.append(dict(name=name, K=K, N=N, qweight=p["qweight"].clone(), lut=p["lut"].clone(),
+                               cheat=p["cheat"], scales=p["scales"], th=p["th"],
+                               out=torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")))
+    xs = {K: F.make_activation(K, g).cuda() for K in {l["K"] for l in layers}}
+    return layers, xs, protos
+
+
+def capture(torch, fn):
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        fn()
+    return graph
+
+
+def time_graph(torch, graph, steps, warmup):
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps * 1e6
+
+
+def roofline_leg(torch, ext, protos, iters=200):
+    """Average duration of the any-precision GEMV kernel on the 4096 -> 14336 shape, HIP events on the
+    stream the kernel is launched on, rotating over private weight copies so each launch reads HBM."""
+    K, N = 4096, 14336
+    p = protos[(K, N)]
+    copies = [p["qweight"].clone() for _ in range(24)]
+    lut = p["lut"]
+    x = torch.randn(1, 1, K, dtype=torch.float16, device="cuda")
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(24):
+            ext.anyprec_gemv(x, out, copies[i], lut, BITS)
+        graph = None
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        for i in range(24):
+            ext.anyprec_gemv(x, out, copies[i], lut, BITS)
+    g.replay(); torch.cuda.synchronize()
+    reps = max(1, iters // 24)
+    with torch.cuda.stream(stream):
+        a = torch.cuda.Event(enable_timing=True); b = torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for _ in range(reps):
+            g.replay()
+        b.record(stream)
+    torch.cuda.synchronize()
+    us = a.elapsed_time(b) * 1e3 / (reps * 24)
+    by = anyprec_bytes(K, N)
+    achieved = by / us / 1e3          # GB/s
+    return {"bound": "hbm", "kernel": "anyprec_kernel<fp16,3> 4096->14336", "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": None}
+
+
+def cpu_baseline_leg(protos, budget_s=15.0):
+    """The same per-layer path (select + residual rows + any-precision GEMV) in the C oracle on the host
+    cores, one layer of each shape, scaled to a token (32 layers)."""
+    import numpy as np
+    from oracle import c_oracle
+    c_oracle.build()
+    cores = os.cpu_count() or 1
+    os.environ.setdefault("OMP_NUM_THREADS", str(min(cores, 64)))
+    rng = np.random.default_rng(0)
+    per_shape = {}
+    t_start = time.perf_counter()
+    for (K, N), p in protos.items():
+        x = rng.standard_normal(K).astype(np.float16)
+        qw = p["qweight"].cpu().numpy(); lut = p["lut"].cpu().numpy()
+        cheat = p["cheat"].numpy(); sc = p["scales"].numpy(); th = p["th"].numpy().astype(np.float32)
+        k = 32 * K // 1024
+        t0 = time.perf_counter()
+        c_oracle.layer_anyprec_dec(x, qw, lut, BITS, cheat, sc, float(th[0]), float(th[k - 1]), 32)
+        per_shape[(K, N)] = (time.perf_counter() - t0) * 1e6
+        if time.perf_counter() - t_start > budget_s:
+            break
+    if len(per_shape) < len(protos):
+        return None
+    token_us = 32 * sum(per_shape[(K, N)] for _, K, N in LLAMA3_8B)
+    return {"value": round(token_us, 1), "unit": "us/token", "cores": int(os.environ["OMP_NUM_THREADS"]),
+            "kind": "port", "sample": "one DEC-compensated layer of each of the 4 Llama-3-8B shapes (C oracle, "
+            "OpenMP, float64 accumulate), x32 layers with q/o, k/v and gate/up counted twice"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32, help="decoder layers per token (32 = Llama-3-8B)")
+    ap.add_argument("--k-chunk", type=int, default=32)
+    ap.add_argument("--n-tb", type=int, default=8)
+    ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from decdec_amd import _lib, ext, formats as F
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    torch.cuda.set_device(0)
+
+    layers, xs, protos = build_layer_set(torch, F, args.layers, args.k_chunk, seed=0)
+    maxK = max(l["K"] for l in layers)
+    rows = torch.zeros(maxK, dtype=torch.int32, device="cuda")
+    acts = torch.zeros(maxK, dtype=torch.float16, device="cuda")
+
+    def make_configs(n_tb, k_chunk):
+        ctx = ext.create_dec_context(n_tb, rows, acts)
+        return ctx, [ext.create_dec_config(ctx, k_chunk, l["cheat"], l["scales"], l["th"]) for l in layers]
+
+    def base_step():
+        for l in layers:
+            l["out"].zero_()
+            ext.anyprec_gemv(xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+
+    ctx, cfgs = make_configs(args.n_tb, args.k_chunk)
+
+    def dec_step():
+        for l, c in zip(layers, cfgs):
+            l["out"].zero_()
+            ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+
+    g_base = capture(torch, base_step)
+    g_dec = capture(torch, dec_step)
+    base_us = time_graph(torch, g_base, args.steps, args.warmup)
+    dec_us = time_graph(torch, g_dec, args.steps, args.warmup)
+    scale = 32.0 / args.layers
+
+    # the zero_() fills are part of the layer contract (APLinear.forward clears its output), so they stay
+    # inside the timed region; their share is reported
+    def zero_step():
+        for l in layers:
+            l["out"].zero_()
+    zero_us = time_graph(torch, capture(torch, zero_step), args.steps, args.warmup)
+
+    weight_bytes = sum(anyprec_bytes(l["K"], l["N"]) for l in layers)
+    host_bytes = sum(args.k_chunk * l["K"] // 1024 * l["N"] // 2 for l in layers)
+    result = {
+        "metric": "us/token over linear layers + DEC slowdown %, Llama-3-8B shapes, batch 1",
+        "value": round(dec_us * scale, 2), "unit": "us/token", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(dec_us / 1e3, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[1]: Llama-3-8B decoder linear shapes, batch 1, any-precision 3-bit base "
+                   "from HBM, 4-bit residuals in pinned host memory", "layers": args.layers,
+                   "linears_per_layer": 7, "k_chunk": args.k_chunk, "n_tb": args.n_tb, "fusion": "single launch",
+                   "graph_replay": True},
+        "base_us_per_token": round(base_us * scale, 2),
+        "dec_slowdown_pct": round((dec_us / base_us - 1) * 100, 2),
+        "zero_fill_us_per_token": round(zero_us * scale, 2),
+        "base_hbm_gbs": round(weight_bytes / (base_us - zero_us) / 1e3, 1),
+        "dec_host_link_bytes_per_token": int(host_bytes * scale),
+    }
+    for c in cfgs:
+        ext.destroy_dec_config(c)
+    ext.destroy_dec_context(ctx)
+
+    if args.sweep:
+        sweep = []
+        for n_tb in (8, 16, 32, 64):
+            for k_chunk in (8, 16, 32, 64):
+                ctx, cfgs = make_configs(n_tb, k_chunk)
+                def step():
+                    for l, c in zip(layers, cfgs):
+                        l["out"].zero_()
+                        ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+                us = time_graph(torch, capture(torch, step), max(5, args.steps // 2), 2)
+                sweep.append({"n_tb": n_tb, "k_chunk": k_chunk, "us_per_token": round(us * scale, 1),
+                              "slowdown_pct": round((us / base_us - 1) * 100, 1)})
+                for c in cfgs:
+                    ext.destroy_dec_config(c)
+                ext.destroy_dec_context(ctx)
+        result["sweep"] = sweep
+
+    result["roofline"] = roofline_leg(torch, ext, protos)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_leg(protos)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -102,13 +102,6 @@ __device__ __forceinline__ uint32_t lane_id() {
 __device__ __forceinline__ uint32_t ballot_rank(unsigned long long m) {
     return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
 }
-// v_writelane_b32: lane `lane` of `old` is replaced by the wave-uniform `val`.  The lane select goes
-// through M0 because gfx9 allows one SGPR on the constant bus per VALU instruction; both scalars come
-// from SALU results here, which needs no software wait states.
-__device__ __forceinline__ uint32_t write_lane(uint32_t old, uint32_t val, int lane) {
-    asm volatile("s_mov_b32 m0, %2\n\tv_writelane_b32 %0, %1, m0" : "+v"(old) : "s"(val), "s"(lane) : "m0");
-    return old;
-}
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);

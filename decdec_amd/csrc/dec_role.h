@@ -151,7 +151,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     uint32_t* key = cnt + 32;                              // [kMaxCand]
     float* cx = (float*)(cnt + 32 + kMaxCand);             // [kMaxCand] (runs into `pre`, unused here)
     uint32_t* pc = (uint32_t*)red;                         // [4][kMaxCand] partial ranks
-    uint32_t T = 0, total = 0, base = 0, bkt = 0;
+    uint32_t total = 0, base = 0, bkt = 0;
     bool fast = false, is_cand = false;
     if (p.monotone) {
         // bucket index = number of floors (up to t2) strictly above |x|
@@ -172,7 +172,6 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
         const bool ok1 = (tot1 >= kc) && (tot1 <= (uint32_t)kMaxCand);
         const bool ok2 = (tot2 >= kc) && (tot2 <= (uint32_t)kMaxCand);
         fast = ok1 || ok2;
-        T = ok1 ? p.t1 : p.t2;
         total = ok1 ? tot1 : tot2;
         const uint32_t excl = incl - v;
         base = (uint32_t)__builtin_amdgcn_readlane((int)excl, (int)(ok1 ? wave : 16u + wave));

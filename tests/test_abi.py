@@ -1,0 +1,80 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/decdec_hip.h declares, and
+its host-only entry points agree with the oracle.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from decdec_amd import _lib
+from oracle import decdec_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "decdec_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(decdec_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 25 and "decdec_dec_anyprec" in names
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/decdec_hip.h but not exported"
+    bound = set(_lib.SIGNATURES) | set(_lib.OTHER_SYMBOLS)
+    assert set(names) == bound, (set(names) ^ bound)
+
+
+def test_version_and_options():
+    lib = _lib.load()
+    assert lib.decdec_version() >= 100
+    assert _lib.get_option("fusion") == 1
+    _lib.set_option("fusion", 0); assert _lib.get_option("fusion") == 0
+    _lib.set_option("fusion", 1)
+    with pytest.raises(RuntimeError, match="unknown option"):
+        _lib.set_option("no_such_option", 1)
+
+
+@pytest.mark.parametrize("dt,code", [("fp16", 1), ("bf16", 2), ("fp32", 0)])
+def test_library_floors_match_oracle_bitwise(dt, code):
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    out = (ctypes.c_float * 32)()
+    for _ in range(500):
+        a = float(O._rounder(dt)(np.float32(abs(rng.standard_normal()) * 10.0 ** rng.integers(-3, 3))))
+        b = float(O._rounder(dt)(np.float32(a * rng.random())))
+        _lib.check(lib.decdec_bucket_floors(a, b, code, out))
+        want = O.bucket_floors(a, b, dt)
+        assert np.array_equal(np.array(out[:], dtype=np.float32).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("K,N,n_tb,k_chunk", [(4096, 4096, 8, 32), (4096, 14336, 16, 32), (5120, 35840, 8, 32),
+                                              (17920, 5120, 16, 64), (28672, 8192, 32, 16), (4096, 1024, 64, 8)])
+def test_library_reference_geometry_matches_oracle(K, N, n_tb, k_chunk):
+    info = _lib.ConfigInfo()
+    _lib.check(_lib.load().decdec_reference_geometry(K, N, n_tb, k_chunk, 1, 65536, ctypes.byref(info)))
+    want = O.dec_geometry(K, N, n_tb, k_chunk, 2, 65536)
+    for key in _lib.REFERENCE_KEYS:
+        assert getattr(info, key) == want[key], key
+
+
+def test_invalid_handles_and_arguments_fail_cleanly():
+    lib = _lib.load()
+    assert lib.decdec_destroy_dec_config(12345) != 0 and "invalid DECConfig handle" in _lib.last_error()
+    assert lib.decdec_destroy_dec_context(12345) != 0 and "invalid DECContext handle" in _lib.last_error()
+    assert lib.decdec_dec(0, None, None, 1, 8, 8, None) != 0
+    h = ctypes.c_uint64(0)
+    assert lib.decdec_create_dec_config(777, 8, 1, None, 0, None, 0, None, 8, 8, ctypes.byref(h)) != 0
+    # plan-time validation of the GEMVs happens before any HIP call
+    buf = (ctypes.c_uint32 * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.decdec_anyprec_gemv(p, p, p, p, 2, 1, 1024, 8, None) != 0 and "Bitwidth must be between 3 and 8" in _lib.last_error()
+    assert lib.decdec_anyprec_gemv(p, p, p, p, 3, 0, 1024, 8, None) != 0 and "does not support float" in _lib.last_error()
+    assert lib.decdec_anyprec_gemv(p, p, p, p, 3, 1, 1000, 8, None) != 0 and "multiple of 32" in _lib.last_error()
+    assert lib.decdec_sqllm_gemv(p, p, p, p, 5, 1, 1024, 8, None) != 0 and "Bitwidth must be 3 or 4" in _lib.last_error()
+    assert lib.decdec_lutgemm_gemv(p, p, p, p, p, 9, 128, 1, 1024, 8, None) != 0 and "between 1 and 8" in _lib.last_error()
+    assert lib.decdec_lutgemm_gemv(p, p, p, p, p, 3, 48, 1, 1024, 8, None) != 0 and "group_size" in _lib.last_error()
