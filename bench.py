@@ -64,10 +64,17 @@ def build_layer_set(torch, F, n_layers, k_chunk, seed):
         for name, K, N in LLAMA3_8B:
             p = protos[(K, N)]
             layers.append(dict(name=name, K=K, N=N, qweight=p["qweight"].clone(), lut=p["lut"].clone(),
-                               cheat=p["cheat"], scales=p["scales"], th=p["th"],
-                               out=torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")))
+                               cheat=p["cheat"], scales=p["scales"], th=p["th"]))
+    # One arena holds every layer's output: the library accumulates into pre-zeroed outputs, and a decode
+    # step that owns its output buffers clears all of them with a single fill instead of one per layer.
+    total = sum((l["N"] + 127) // 128 * 128 for l in layers)
+    arena = torch.zeros(total, dtype=torch.float16, device="cuda")
+    off = 0
+    for l in layers:
+        l["out"] = arena[off:off + l["N"]].view(1, 1, l["N"])
+        off += (l["N"] + 127) // 128 * 128
     xs = {K: F.make_activation(K, g).cuda() for K in {l["K"] for l in layers}}
-    return layers, xs, protos
+    return layers, xs, protos, arena
 
 
 def capture(torch, fn):
@@ -92,40 +99,57 @@ def time_graph(torch, graph, steps, warmup):
     return (time.perf_counter() - t0) / steps * 1e6
 
 
-def roofline_leg(torch, ext, protos, iters=200):
+# HBM traffic of one launch of the roofline kernel, bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --leg roofline`, each scaled by what the same counter reads for the 256 MiB device copy that the
+# leg also runs (profiles/anyprec_gemv_4096x14336_pmc.md holds the runs); None = not measured for this build
+MEASURED_TRAFFIC = {"anyprec_kernel<fp16,3> 4096->14336": 23111000}
+
+
+def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
     """Average duration of the any-precision GEMV kernel on the 4096 -> 14336 shape, HIP events on the
     stream the kernel is launched on, rotating over private weight copies so each launch reads HBM."""
     K, N = 4096, 14336
     p = protos[(K, N)]
-    copies = [p["qweight"].clone() for _ in range(24)]
+    ncopy = 24
+    copies = [p["qweight"].clone() for _ in range(ncopy)]
     lut = p["lut"]
     x = torch.randn(1, 1, K, dtype=torch.float16, device="cuda")
     out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
     stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        for i in range(24):
+
+    def launches():
+        for i in range(ncopy):
             ext.anyprec_gemv(x, out, copies[i], lut, BITS)
-        graph = None
+    with torch.cuda.stream(stream):
+        launches()
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g, stream=stream):
-        for i in range(24):
-            ext.anyprec_gemv(x, out, copies[i], lut, BITS)
-    g.replay(); torch.cuda.synchronize()
-    reps = max(1, iters // 24)
+        launches()
+    g.replay()
+    torch.cuda.synchronize()
+    reps = max(1, iters // ncopy)
     with torch.cuda.stream(stream):
-        a = torch.cuda.Event(enable_timing=True); b = torch.cuda.Event(enable_timing=True)
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
         a.record(stream)
         for _ in range(reps):
             g.replay()
         b.record(stream)
     torch.cuda.synchronize()
-    us = a.elapsed_time(b) * 1e3 / (reps * 24)
+    us = a.elapsed_time(b) * 1e3 / (reps * ncopy)
+    if calibrate_copy:      # known-size device copy for scaling the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     by = anyprec_bytes(K, N)
     achieved = by / us / 1e3          # GB/s
-    return {"bound": "hbm", "kernel": "anyprec_kernel<fp16,3> 4096->14336", "achieved": round(achieved, 1),
+    name = "anyprec_kernel<fp16,3> 4096->14336"
+    return {"bound": "hbm", "kernel": name, "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": None}
+            "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": MEASURED_TRAFFIC.get(name)}
 
 
 def cpu_baseline_leg(protos, budget_s=15.0):
@@ -167,6 +191,8 @@ def main():
     ap.add_argument("--n-tb", type=int, default=8)
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--leg", choices=["all", "roofline"], default="all",
+                    help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter collection)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
@@ -178,7 +204,11 @@ def main():
     _lib.load()
     torch.cuda.set_device(0)
 
-    layers, xs, protos = build_layer_set(torch, F, args.layers, args.k_chunk, seed=0)
+    if args.leg == "roofline":
+        _, _, protos, _ = build_layer_set(torch, F, 0, args.k_chunk, seed=0)
+        print(json.dumps({"roofline": roofline_leg(torch, ext, protos, iters=48, calibrate_copy=True)}))
+        return
+    layers, xs, protos, arena = build_layer_set(torch, F, args.layers, args.k_chunk, seed=0)
     maxK = max(l["K"] for l in layers)
     rows = torch.zeros(maxK, dtype=torch.int32, device="cuda")
     acts = torch.zeros(maxK, dtype=torch.float16, device="cuda")
@@ -188,15 +218,15 @@ def main():
         return ctx, [ext.create_dec_config(ctx, k_chunk, l["cheat"], l["scales"], l["th"]) for l in layers]
 
     def base_step():
+        arena.zero_()
         for l in layers:
-            l["out"].zero_()
             ext.anyprec_gemv(xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
 
     ctx, cfgs = make_configs(args.n_tb, args.k_chunk)
 
     def dec_step():
+        arena.zero_()
         for l, c in zip(layers, cfgs):
-            l["out"].zero_()
             ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
 
     g_base = capture(torch, base_step)
@@ -205,12 +235,9 @@ def main():
     dec_us = time_graph(torch, g_dec, args.steps, args.warmup)
     scale = 32.0 / args.layers
 
-    # the zero_() fills are part of the layer contract (APLinear.forward clears its output), so they stay
-    # inside the timed region; their share is reported
-    def zero_step():
-        for l in layers:
-            l["out"].zero_()
-    zero_us = time_graph(torch, capture(torch, zero_step), args.steps, args.warmup)
+    # clearing the outputs is part of the layer contract (the kernels accumulate), so the arena fill stays
+    # inside the timed region; its share is reported
+    zero_us = time_graph(torch, capture(torch, lambda: arena.zero_()), args.steps, args.warmup)
 
     weight_bytes = sum(anyprec_bytes(l["K"], l["N"]) for l in layers)
     host_bytes = sum(args.k_chunk * l["K"] // 1024 * l["N"] // 2 for l in layers)
@@ -239,8 +266,8 @@ def main():
             for k_chunk in (8, 16, 32, 64):
                 ctx, cfgs = make_configs(n_tb, k_chunk)
                 def step():
+                    arena.zero_()
                     for l, c in zip(layers, cfgs):
-                        l["out"].zero_()
                         ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
                 us = time_graph(torch, capture(torch, step), max(5, args.steps // 2), 2)
                 sweep.append({"n_tb": n_tb, "k_chunk": k_chunk, "us_per_token": round(us * scale, 1),

@@ -1,6 +1,7 @@
 // C-ABI layer of libdecdec_hip.so: argument validation, DEC context / config objects, launch
 // planning, and the two ways of running DEC next to a base GEMV (one fused launch, or the
 // reference's two-stream fork/join).  Declarations and reference citations: include/decdec_hip.h.
+#include <cmath>
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -223,7 +224,7 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, DecPlan*
         const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
         for (uint32_t sg = 1; sg <= sg_max; ++sg) {
             const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
-            const uint32_t slots = cpb * std::max(k_chunk, 1u);
+            const uint32_t slots = (cpb * std::max(k_chunk, 1u) + 1u) & ~1u;   // even: keeps the LDS arrays behind the row list 16-byte aligned
             const size_t lds = dec_lds_bytes(slots);
             if (lds > kLdsBudget) continue;
             // per-workgroup critical path: sequential chunk selections, then batches of eight rows per
@@ -238,7 +239,7 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, DecPlan*
     if (best_cg == 0) return 1;
     pl->cg = best_cg; pl->sg = best_sg; pl->nseg = nseg; pl->vec = 1;
     pl->segs_per_block = cdiv(nseg, best_sg);
-    pl->slots = cdiv(num_chunks, best_cg) * std::max(k_chunk, 1u);
+    pl->slots = (cdiv(num_chunks, best_cg) * std::max(k_chunk, 1u) + 1u) & ~1u;
     pl->lds_reduce = 1; pl->lds = best_lds;
     return 0;
 }
@@ -278,10 +279,9 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
         const float a = load_host(c->thresholds_host, c->dt, 0);
         const float b = load_host(c->thresholds_host, c->dt, (size_t)k - 1);
         bucket_floors(a, b, c->dt, p->floors);
-        bool mono = p->floors[0] == p->floors[0];
+        bool mono = std::isfinite(p->floors[0]) && std::isfinite(p->floors[kBuckets - 1]);
         for (int i = 1; i < kBuckets; ++i) mono = mono && (p->floors[i] <= p->floors[i - 1]);
         p->monotone = mono ? 1u : 0u;
-        p->t1 = 18; p->t2 = 24;
     }
     p->K = c->K; p->N = c->N; p->M = c->M;
     p->num_chunks = cdiv(c->K, 1024); p->k_chunk = c->k_chunk; p->k_total = (uint32_t)k;

@@ -31,8 +31,7 @@ struct DecParams {
     void* sel_acts;             // context scratch: selected activations
     void* out;                  // output [N], accumulated atomically
     float floors[kBuckets];     // bucket floors (values exactly representable in the activation dtype)
-    uint32_t monotone;          // floors are non-increasing and free of NaN (enables the fast selection path)
-    uint32_t t1, t2;            // last bucket considered by the first / second fast-path attempt
+    uint32_t monotone;          // floors are finite and non-increasing (enables the fast selection path)
     uint32_t K, N, M;           // M = N / 8 words per residual row
     uint32_t num_chunks, k_chunk, k_total;
     uint32_t cg, sg;            // chunk groups x segment groups = number of DEC workgroups
@@ -63,11 +62,16 @@ __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots) {
 // floors (non-monotone floors can put a channel into several buckets, as in the reference kernel).
 template <int DT>
 __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t c, uint32_t t_local, uint32_t kc,
-                                                float a, float xv, float myfloor, int32_t* lrows, float* lacts,
-                                                uint32_t* cnt, uint32_t* pre, bool write_global) {
+                                                int32_t* lrows, float* lacts, uint32_t* cnt, uint32_t* pre,
+                                                bool write_global) {
     using E = Elem<DT>;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t lo = c * kChunk;
+    const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
+    const bool in = tid < len;
+    const float xv = in ? E::load(p.x, lo + tid) : 0.f;
+    const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");   // NaN is a member of no bucket
+    const float myfloor = p.floors[lane & 31u];                      // lane i holds floor[i]
     uint32_t member = 0;
     float ce = __builtin_inff();
 #pragma unroll 1
@@ -115,95 +119,153 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
     }
 }
 
-// Inclusive prefix sum over each group of 16 lanes (DPP row shifts, zero fill).
-__device__ __forceinline__ uint32_t row_scan16(uint32_t v) {
+// Inclusive prefix sum over the 64 lanes of a wave (DPP row shifts and row broadcasts, zero fill).
+__device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
     v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, true);   // row_shr 1
     v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, true);   // row_shr 2
     v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, true);   // row_shr 4
     v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, true);   // row_shr 8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, true);   // row_bcast 15 -> rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, true);   // row_bcast 31 -> rows 2, 3
     return v;
 }
 
-// Fast path (floors non-increasing and free of NaN, checked on the host).  Then bucket(|x|) is the
-// number of floors above |x|, buckets 0..T tile [floor_T, +inf), and as soon as at least kc channels lie
-// in that range they are the only possible picks.  Those candidates (usually a few dozen of 1024) are
-// compacted in channel order with the key (bucket << 10 | channel); the canonical position of a
-// candidate is the number of smaller keys, counted all-pairs by the whole workgroup.  No sequential
-// walk over buckets, so the latency is a handful of LDS round trips.
+// Fast path (floors finite and non-increasing, checked on the host).  Then bucket(|x|) is the number of
+// floors above |x|, buckets 0..T tile [floor_T, +inf), and as soon as at least kc channels lie in that
+// range they are the only possible picks.  Eight cut-offs T are tried at once (a compare and a ballot
+// each); the first whose range holds at least kc and at most kMaxCand channels wins.  Those candidates
+// (usually a few dozen of 1024) are compacted in channel order, get the key (bucket << 10 | channel),
+// and the canonical position of a candidate is the number of smaller keys, counted all-pairs in tiles of
+// 64 candidates x 16 keys spread over the waves.  No sequential walk over buckets.
+//
+// A wave issues one instruction every four cycles whatever its kind, and an instruction issued by all
+// 16 waves of the workgroup occupies each SIMD four times as long; so the scan of the 1024 channels is
+// done by four waves (one per SIMD, four channels per lane) while the others wait at the barrier, and
+// the candidate phases only involve the waves that hold candidates or tiles.
+constexpr int kAttempts = 8;
+constexpr int kSelWaves = 4;
+__device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) {
+    return u == 0 ? 15u : u == 1 ? 18u : u == 2 ? 21u : u == 3 ? 23u : u == 4 ? 25u : u == 5 ? 27u : u == 6 ? 29u : 31u;
+}
+
 template <int DT>
 __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
                                                  int32_t* lrows, float* lacts, uint32_t* cnt,
                                                  uint32_t* pre, float* red, bool write_global) {
     using E = Elem<DT>;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lo = c * kChunk;
     const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
     const uint32_t kc = p.k_chunk * len / kChunk;
     if (kc == 0) return;                                   // uniform for the workgroup
 
-    const bool in = tid < len;
-    const float xv = in ? E::load(p.x, lo + tid) : 0.f;
-    const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");   // NaN is a member of no bucket
-    const float myfloor = p.floors[lane & 31u];            // lane i holds floor[i]
-    dec_stamp(p, blockIdx.x, 5);
-
-    uint32_t* wc = cnt;                                    // [2][16] candidate counts per wave
+    uint32_t* wc = cnt;                                    // [kAttempts][kSelWaves] candidate counts
     uint32_t* key = cnt + 32;                              // [kMaxCand]
     float* cx = (float*)(cnt + 32 + kMaxCand);             // [kMaxCand] (runs into `pre`, unused here)
-    uint32_t* pc = (uint32_t*)red;                         // [4][kMaxCand] partial ranks
-    uint32_t total = 0, base = 0, bkt = 0;
-    bool fast = false, is_cand = false;
-    if (p.monotone) {
-        // bucket index = number of floors (up to t2) strictly above |x|
-#pragma unroll 1
-        for (uint32_t i = 0; i <= p.t2; ++i) {
-            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), (int)i));
-            bkt += (a < fl) ? 1u : 0u;
+    uint32_t* hdr = cnt + 32 + 2 * kMaxCand;               // fast flag, candidate count
+    uint32_t* pc = (uint32_t*)red;                         // [16][kMaxCand] partial ranks
+    const bool scanner = p.monotone && wave < (uint32_t)kSelWaves;   // uniform per wave
+
+    // ---- four waves scan the chunk: lane l of wave w owns channels 4 (64 w + l) .. + 3
+    float xv[4], a[4];
+    const uint32_t ch0 = 4u * tid;
+    if (scanner) {
+        // unconditional loads from clamped indices (a predicated load costs a branch and a full wait each)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) xv[s] = E::load(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const bool in = ch0 + s < len;
+            const float v = __builtin_fabsf(xv[s]);
+            a[s] = (in && v < __builtin_inff()) ? v : -__builtin_inff();   // NaN, inf: members of no bucket
         }
-        const bool finite = a < __builtin_inff();          // false for NaN and inf
-        const bool c1 = finite && (bkt <= p.t1), c2 = finite && (bkt <= p.t2);
-        const unsigned long long m1 = __ballot(c1), m2 = __ballot(c2);
-        if (lane == 0) { wc[wave] = (uint32_t)__popcll(m1); wc[16 + wave] = (uint32_t)__popcll(m2); }
-        __syncthreads();
-        const uint32_t v = wc[lane & 31u];                 // lanes 0..15: first attempt, 16..31: second
-        const uint32_t incl = row_scan16(v);
-        const uint32_t tot1 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 15);
-        const uint32_t tot2 = (uint32_t)__builtin_amdgcn_readlane((int)incl, 31);
-        const bool ok1 = (tot1 >= kc) && (tot1 <= (uint32_t)kMaxCand);
-        const bool ok2 = (tot2 >= kc) && (tot2 <= (uint32_t)kMaxCand);
-        fast = ok1 || ok2;
-        total = ok1 ? tot1 : tot2;
-        const uint32_t excl = incl - v;
-        base = (uint32_t)__builtin_amdgcn_readlane((int)excl, (int)(ok1 ? wave : 16u + wave));
-        is_cand = ok1 ? c1 : c2;
-        if (fast) {
-            const unsigned long long cm = ok1 ? m1 : m2;
-            if (is_cand) {
-                const uint32_t idx = base + ballot_rank(cm);
-                key[idx] = (bkt << 10) | tid;
-                cx[idx] = xv;
-            }
+        dec_stamp(p, blockIdx.x, 5);
+        uint32_t n[kAttempts];
+#pragma unroll
+        for (int u = 0; u < kAttempts; ++u) {
+            const float f = p.floors[dec_attempt_bucket(u)];
+            n[u] = 0;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) n[u] += (uint32_t)__popcll(__ballot(a[s] >= f));
         }
-        __syncthreads();
-    }
-    if (!fast) {
-        dec_select_general<DT>(p, c, t_local, kc, a, xv, myfloor, lrows, lacts, cnt, pre, write_global);
-        return;
-    }
-    dec_stamp(p, blockIdx.x, 6);
-    {   // partial rank of candidate j among candidates [64 q, 64 q + 64)
-        const uint32_t j = tid & (uint32_t)(kMaxCand - 1), q = tid / (uint32_t)kMaxCand;
-        const uint32_t mykey = j < total ? key[j] : 0u;
-        const uint32_t q0 = q * 64u;
-        const uint32_t qn = q0 >= total ? 0u : ((total - q0) < 64u ? (total - q0) : 64u);
-        uint32_t r = 0;
-#pragma unroll 4
-        for (uint32_t it = 0; it < qn; ++it) r += (key[q0 + it] < mykey) ? 1u : 0u;
-        pc[q * kMaxCand + j] = r;
+        if (lane == 0) {
+#pragma unroll
+            for (int u = 0; u < kAttempts; ++u) wc[u * kSelWaves + wave] = n[u];
+        }
     }
     __syncthreads();
-    if (tid < total) {
-        const uint32_t pos = pc[tid] + pc[kMaxCand + tid] + pc[2 * kMaxCand + tid] + pc[3 * kMaxCand + tid];
+    if (scanner) {
+        // lane u < 8 looks at attempt u: total and the count of the waves before this one
+        const u32x4 w4 = *(const u32x4*)(wc + kSelWaves * (lane & 7u));
+        const uint32_t tot = w4[0] + w4[1] + w4[2] + w4[3];
+        const uint32_t before = (wave > 0 ? w4[0] : 0u) + (wave > 1 ? w4[1] : 0u) + (wave > 2 ? w4[2] : 0u);
+        const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= (uint32_t)kMaxCand);
+        const bool fast = okm != 0ull;
+        if (fast) {
+            const uint32_t us = (uint32_t)__builtin_ctzll(okm);                     // first qualifying attempt
+            const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)us);
+            const uint32_t base = (uint32_t)__builtin_amdgcn_readlane((int)before, (int)us);
+            const float f = p.floors[dec_attempt_bucket(us)];
+            uint32_t cs[4], mine = 0;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) { cs[s] = (a[s] >= f) ? 1u : 0u; mine += cs[s]; }
+            uint32_t idx = base + wave_scan(mine) - mine;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
+            }
+            if (tid == 0) hdr[1] = total;
+        }
+        if (tid == 0) hdr[0] = fast ? 1u : 0u;
+    } else if (!p.monotone && tid == 0) {
+        hdr[0] = 0u;
+    }
+    __syncthreads();
+    const u32x2 hd = *(const u32x2*)hdr;
+    if (hd[0] == 0u) {                                     // uniform
+        __syncthreads();                                   // hdr is read before cnt is reused
+        dec_select_general<DT>(p, c, t_local, kc, lrows, lacts, cnt, pre, write_global);
+        return;
+    }
+    const uint32_t total = hd[1];
+    dec_stamp(p, blockIdx.x, 6);
+    // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
+    if (__builtin_amdgcn_readfirstlane(tid & ~63u) < total) {
+        if (tid < total) {
+            const float ca = __builtin_fabsf(cx[tid]);
+            uint32_t bkt = 0;
+#pragma unroll
+            for (int i = 0; i < kBuckets; ++i) bkt += (ca < p.floors[i]) ? 1u : 0u;
+            key[tid] |= bkt << 10;
+        } else if (tid < ((total + 15u) & ~15u)) {
+            key[tid] = 0xFFFFFFFFu;                        // padding of the last 16-key tile: never smaller
+        }
+    }
+    __syncthreads();
+    {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per wave and round
+        const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
+#pragma unroll 1
+        for (uint32_t tile = wave; tile < ntiles; tile += kDecWaves) {
+            const uint32_t jg = tile % njg, iq = tile / njg;
+            const uint32_t j = jg * 64u + lane;
+            const uint32_t mykey = j < total ? key[j] : 0u;
+            const u32x4* kp = (const u32x4*)(key + iq * 16u);
+            uint32_t r = 0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const u32x4 k4 = kp[v];
+                r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
+            }
+            pc[iq * kMaxCand + j] = r;
+        }
+    }
+    __syncthreads();
+    if (__builtin_amdgcn_readfirstlane(tid & ~63u) < total && tid < total) {
+        const uint32_t niq = (total + 15u) >> 4;
+        uint32_t pos = 0;
+#pragma unroll 4
+        for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kMaxCand + tid];
         if (pos < kc) {
             const uint32_t ch = lo + (key[tid] & 1023u);
             const float xs = cx[tid];
