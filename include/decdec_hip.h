@@ -42,7 +42,7 @@ typedef struct decdec_config_info {
     int32_t hip_dec_blocks;        /* workgroups of 1024 threads given to DEC (<= num_tb) */
     int32_t hip_chunk_groups;      /* = atomic adds each output receives from DEC */
     int32_t hip_segment_groups;
-    int32_t hip_vec_words;         /* u32 words per lane per residual load: 1, 2, 4 */
+    int32_t hip_vec_words;         /* u32 words per lane per residual load (always 1: 256-byte wave loads) */
     int32_t hip_lds_bytes;
     int32_t hip_slots_per_block;
     int32_t hip_lds_reduce;
@@ -97,8 +97,8 @@ int decdec_unfused_dec(uint64_t config, const void* input, void* output, int dty
                        uint32_t in_features, uint32_t out_features, void* stream);
 
 /* anyprec_gemv (decdec.cu:324-333 -> matmul_kbit_32 anyprec.cu:344-514). qweight int32
- * [>=bitwidth, out, in/32] (only the first `bitwidth` planes are read; `qweight_planes` is the
- * allocated plane count), lut `dtype`[out, 2^bitwidth]; fp16 / bf16 only; bitwidth 3..8. */
+ * [>=bitwidth, out, in/32] (only the first `bitwidth` planes are read; plane p starts at word
+ * p*out*in/32), lut `dtype`[out, 2^bitwidth]; fp16 / bf16 only; bitwidth 3..8. */
 int decdec_anyprec_gemv(const void* input, void* output, const void* qweight, const void* lut,
                         int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
                         void* stream);
