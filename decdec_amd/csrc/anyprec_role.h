@@ -31,6 +31,8 @@ struct AnyprecParams {
     uint32_t rg;           // row groups per workgroup
     uint32_t rpw;          // rows per wave: 2, 4 or 8, all in flight together
     uint32_t x_aligned;    // activation pointer is 16-byte aligned
+    // tile decoder (3-bit, K a multiple of 1024): waves per tile (0 = not used), K-tiles per row group, tiles
+    uint32_t tile_cs, tile_kt, tiles;
 };
 
 __host__ __device__ inline size_t anyprec_lds_bytes(uint32_t S, uint32_t rg, uint32_t rpw, int bits) {
@@ -76,35 +78,41 @@ __device__ __forceinline__ void anyprec_arrange_x(const uint32_t (&xr)[4][4], ui
     }
 }
 
+// Bit masks of the 3-bit decoder, kept in VGPRs: a VALU operation whose sources are all VGPRs (or inline
+// constants) issues at twice the rate of one that reads an SGPR or a 32-bit literal.
+struct Anyprec3Masks {
+    uint32_t m8, m4, m2, k7;
+    __device__ __forceinline__ void init() {
+        m8 = 0x88888888u; m4 = 0x44444444u; m2 = 0x22222222u; k7 = 0x07070707u;
+        asm volatile("" : "+v"(m8), "+v"(m4), "+v"(m2), "+v"(k7));
+    }
+};
+// bits of a where m is set, bits of b elsewhere (one three-input bit operation)
+__device__ __forceinline__ uint32_t bit_select(uint32_t m, uint32_t a, uint32_t b) { return ((a ^ b) & m) ^ b; }
+
 // One word of a 3-bit row: 32 weights looked up through byte-permutes and dotted with xp.
-// lut4 holds the row's eight 16-bit LUT entries (two per dword).
+// lo0/lo1/hi0/hi1 are the row's byte tables: LO = low bytes of LUT entries 0..7, HI = high bytes.
 template <int DT>
-__device__ __forceinline__ float anyprec3_word(uint32_t q0, uint32_t q1, uint32_t q2, const u32x4 lut4,
+__device__ __forceinline__ float anyprec3_word(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t lo0, uint32_t lo1,
+                                               uint32_t hi0, uint32_t hi1, const Anyprec3Masks& mk,
                                                const uint32_t (&xp)[8][2], float acc) {
-    // byte tables: LO = low bytes of entries 0..7, HI = high bytes
-    const uint32_t lo0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x06040200u);
-    const uint32_t hi0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x07050301u);
-    const uint32_t lo1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x06040200u);
-    const uint32_t hi1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x07050301u);
-    // index words: nibble n of T_o carries the 3-bit index of bit 4n+o (o = 3..0), either at nibble
-    // bits 3..1 (T3, T1) or 2..0 (T2, T0); the unused nibble bit is garbage and masked below.
+    // index words: nibble n of T_o carries the 3-bit index of bit 4n+o (o = 3..0) at nibble bits 2..0; the
+    // fourth nibble bit is garbage and masked below.
     const uint32_t r1 = q1 >> 1, r2 = q2 >> 2, l0 = q0 << 2, l1 = q1 << 1;
-    const uint32_t m8 = 0x88888888u, m4 = 0x44444444u, m2 = 0x22222222u;
-    const uint32_t t3 = (q0 & m8) | (r1 & m4) | (r2 & ~(m8 | m4));
-    const uint32_t t2 = (q0 & m4) | (r1 & m2) | (r2 & ~(m4 | m2));
-    const uint32_t t1 = (l0 & m8) | (l1 & m4) | (q2 & ~(m8 | m4));
-    const uint32_t t0 = (l0 & m4) | (l1 & m2) | (q2 & ~(m4 | m2));
-    const uint32_t k7 = 0x07070707u;
+    const uint32_t t3 = bit_select(mk.m8, q0, bit_select(mk.m4, r1, r2)) >> 1;
+    const uint32_t t2 = bit_select(mk.m4, q0, bit_select(mk.m2, r1, r2));
+    const uint32_t t1 = bit_select(mk.m8, l0, bit_select(mk.m4, l1, q2)) >> 1;
+    const uint32_t t0 = bit_select(mk.m4, l0, bit_select(mk.m2, l1, q2));
     // selector bytes 0..3 <-> j = 3..0; element e per selector as listed
     const uint32_t sel[8] = {
-        (t3 >> 5) & k7,   // e = 0
-        (t2 >> 4) & k7,   // e = 1
-        (t1 >> 5) & k7,   // e = 2
-        (t0 >> 4) & k7,   // e = 3
-        (t3 >> 1) & k7,   // e = 4
-        t2 & k7,          // e = 5
-        (t1 >> 1) & k7,   // e = 6
-        t0 & k7,          // e = 7
+        (t3 >> 4) & mk.k7,   // e = 0
+        (t2 >> 4) & mk.k7,   // e = 1
+        (t1 >> 4) & mk.k7,   // e = 2
+        (t0 >> 4) & mk.k7,   // e = 3
+        t3 & mk.k7,          // e = 4
+        t2 & mk.k7,          // e = 5
+        t1 & mk.k7,          // e = 6
+        t0 & mk.k7,          // e = 7
     };
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -116,6 +124,13 @@ __device__ __forceinline__ float anyprec3_word(uint32_t q0, uint32_t q1, uint32_
         acc = dot2_acc<DT>(w10, xp[e][1], acc);
     }
     return acc;
+}
+// byte tables of a row's eight 16-bit LUT entries (two per dword of lut4)
+__device__ __forceinline__ void anyprec3_tables(const u32x4 lut4, uint32_t& lo0, uint32_t& lo1, uint32_t& hi0, uint32_t& hi1) {
+    lo0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x06040200u);
+    hi0 = __builtin_amdgcn_perm(lut4[1], lut4[0], 0x07050301u);
+    lo1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x06040200u);
+    hi1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x07050301u);
 }
 
 // Generic bit width: indices assembled bytewise, weights from a per-wave LDS copy of the LUT (fp32).
@@ -216,11 +231,15 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
             for (int e = 0; e < 8; ++e) { xp[e][0] = 0u; xp[e][1] = 0u; }
         }
         float sums[RB];
+        Anyprec3Masks mk;
+        mk.init();
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             float acc;
             if constexpr (BITS == 3) {
-                acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lut4[r], xp, 0.f);
+                uint32_t lo0, lo1, hi0, hi1;
+                anyprec3_tables(lut4[r], lo0, lo1, hi0, hi1);
+                acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lo0, lo1, hi0, hi1, mk, xp, 0.f);
             } else {
                 constexpr int L = 1 << BITS;
                 const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
@@ -261,8 +280,106 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
     }
 }
 
+// ---- 3-bit tile decoder -----------------------------------------------------------------------------
+// The decode above spends a fifth of its vector instructions on work that exists only because the 64
+// lanes of a wave share a row: rearranging the activations per lane, building the row's byte tables in
+// every lane, and the cross-lane sum.  Here a lane owns a ROW instead.  A tile is 64 rows x (4 CS) words;
+// its 3 planes are loaded with coalesced 16-byte requests (16 CS bytes of a row per CS lanes), staged in
+// LDS with a padded pitch, and read back transposed: wave `wq` of the tile reads, for its lane's row, the
+// four words 4 wq .. 4 wq + 3 of every plane in three conflict-free 16-byte LDS reads.  The activations
+// of those words are the same for all 64 rows, so they arrive through the scalar cache and stay in SGPRs;
+// the byte tables are built once per wave; every lane ends with its row's partial sum, the CS waves of a
+// tile are added in LDS and one atomic per output pair and tile goes to memory (K / (128 CS) per output).
+__host__ __device__ inline size_t anyprec3_tile_lds_bytes(uint32_t cs) {
+    return (size_t)3 * 64 * (cs * 16 + 16) + (size_t)cs * 64 * 4;
+}
+
+template <int DT>
+__device__ __forceinline__ void anyprec3_tile(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
+    using E = Elem<DT>;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t CS = p.tile_cs;
+    const uint32_t sub = wave / CS, wq = wave % CS;
+    const uint32_t g = bid * ((blockDim.x >> 6) / CS) + sub;             // global tile index
+    const bool tile_ok = g < p.tiles;                                    // uniform per wave
+    const uint32_t gg = tile_ok ? g : 0u;
+    const uint32_t rgi = gg / p.tile_kt, kt = gg % p.tile_kt;
+    const uint32_t row0 = rgi * 64u, w0 = kt * 4u * CS;
+    const uint32_t pitch = CS * 16u + 16u;
+    unsigned char* lds = smem + (size_t)sub * anyprec3_tile_lds_bytes(CS);
+    float* part = (float*)(lds + (size_t)3 * 64 * pitch);
+
+    // -- stage the tile: thread tt of the tile loads 16 bytes of row tt / CS, column tt % CS, per plane
+    {
+        const uint32_t tt = wq * 64u + lane, r = tt / CS, c = tt % CS;
+        const uint32_t row = (row0 + r < p.N) ? row0 + r : p.N - 1u;     // rows past the end re-read the last row
+        const uint32_t* src = p.qweight + (size_t)row * p.W + w0 + 4u * c;
+        const size_t plane_stride = (size_t)p.N * p.W;
+        u32x4 v[3];
+#pragma unroll
+        for (int pl = 0; pl < 3; ++pl) v[pl] = __builtin_nontemporal_load((const u32x4*)(src + pl * plane_stride));
+#pragma unroll
+        for (int pl = 0; pl < 3; ++pl) *(u32x4*)(lds + (size_t)pl * 64 * pitch + r * pitch + 16u * c) = v[pl];
+    }
+    // -- this lane's row: LUT byte tables
+    const uint32_t myrow = (row0 + lane < p.N) ? row0 + lane : p.N - 1u;
+    const u32x4 lut4 = *(const u32x4*)((const uint16_t*)p.lut + (size_t)myrow * 8);
+    uint32_t lo0, lo1, hi0, hi1;
+    anyprec3_tables(lut4, lo0, lo1, hi0, hi1);
+    // -- activations of the wave's four words: 16 consecutive dwords per channel group j, scalar loads
+    const uint32_t wfirst = w0 + 4u * wq;                                // first word of this wave
+    const uint32_t ci = wfirst >> 5, tf = wfirst & 31u;                  // chunk, word inside the chunk
+    const DD_CONST_AS uint32_t* xs = (const DD_CONST_AS uint32_t*)p.x + (512u * ci + 4u * tf);
+    uint32_t X[4][16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int d = 0; d < 16; ++d) X[j][d] = xs[128 * j + d];
+    Anyprec3Masks mk;
+    mk.init();
+    __syncthreads();
+    float acc = 0.f;
+    {
+        u32x4 q[3];
+#pragma unroll
+        for (int pl = 0; pl < 3; ++pl) q[pl] = *(const u32x4*)(lds + (size_t)pl * 64 * pitch + lane * pitch + 16u * wq);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            uint32_t xp[8][2];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t x3 = X[3][4 * k + (e >> 1)], x2 = X[2][4 * k + (e >> 1)];
+                const uint32_t x1 = X[1][4 * k + (e >> 1)], x0 = X[0][4 * k + (e >> 1)];
+                if (e & 1) {
+                    xp[e][0] = (x3 >> 16) | (x2 & 0xFFFF0000u);          // lo = j3, hi = j2
+                    xp[e][1] = (x1 >> 16) | (x0 & 0xFFFF0000u);          // lo = j1, hi = j0
+                } else {
+                    xp[e][0] = (x3 & 0xFFFFu) | (x2 << 16);
+                    xp[e][1] = (x1 & 0xFFFFu) | (x0 << 16);
+                }
+            }
+            acc = anyprec3_word<DT>(q[0][k], q[1][k], q[2][k], lo0, lo1, hi0, hi1, mk, xp, acc);
+        }
+    }
+    part[wq * 64u + lane] = acc;
+    __syncthreads();
+    if (wq == 0 && lane < 32u && tile_ok) {
+        const uint32_t r = 2u * lane, row = row0 + r;
+        if (row < p.N) {
+            float v0 = 0.f, v1 = 0.f;
+            for (uint32_t w = 0; w < CS; ++w) { v0 += part[w * 64u + r]; v1 += part[w * 64u + r + 1u]; }
+            if (row + 1u < p.N) E::atomic_add2(p.out, row, v0, v1);
+            else E::atomic_add1(p.out, row, v0);
+        }
+    }
+}
+
 template <int DT, int BITS>
 __device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bid, unsigned char* smem) {
+    if constexpr (BITS == 3) {
+        if (p.tile_cs != 0u) { anyprec3_tile<DT>(p, bid, smem); return; }
+    }
     if (p.rpw == 8) anyprec_rows<DT, BITS, 8>(p, bid, smem);
     else if (p.rpw == 4) anyprec_rows<DT, BITS, 4>(p, bid, smem);
     else anyprec_rows<DT, BITS, 2>(p, bid, smem);

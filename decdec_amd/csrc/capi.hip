@@ -53,6 +53,7 @@ struct Options {
     int sqllm_ktiles = 0;
     int dec_trace = 0;
     int anyprec_rg = 0;
+    int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
 // Diagnostics: per-workgroup cycle stamps of the DEC phases (option "dec_trace").
@@ -68,6 +69,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "sqllm_ktiles")) return &g_opt.sqllm_ktiles;
     if (!strcmp(name, "dec_trace")) return &g_opt.dec_trace;
     if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
+    if (!strcmp(name, "anyprec_tile")) return &g_opt.anyprec_tile;
     return nullptr;
 }
 
@@ -343,6 +345,20 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     pl->d.grid = cdiv(N, p.rg * p.rpw) * p.sgroups;
     pl->d.block = fused_block ? 1024u : 64u * p.S * p.rg;
     pl->d.lds = anyprec_lds_bytes(p.S, p.rg, p.rpw, bits);
+    // 3-bit tile decoder: needs whole 1024-channel chunks, 16-byte aligned planes and LUT rows, and a
+    // dword-aligned activation vector (it is read through the scalar cache)
+    const bool tile_able = bits == 3 && K % 1024 == 0 && ((uintptr_t)qweight % 16) == 0 &&
+                           ((uintptr_t)input % 4) == 0 && g_opt.anyprec_tile != 0;
+    if (tile_able) {
+        const uint32_t cs = (g_opt.anyprec_tile == 2 || g_opt.anyprec_tile == 4) ? (uint32_t)g_opt.anyprec_tile : 8u;
+        p.tile_cs = cs;
+        p.tile_kt = p.W / (4u * cs);
+        p.tiles = cdiv(N, 64) * p.tile_kt;
+        const uint32_t waves = fused_block ? 16u : cs;
+        pl->d.block = 64u * waves;
+        pl->d.grid = cdiv(p.tiles, waves / cs);
+        pl->d.lds = (waves / cs) * anyprec3_tile_lds_bytes(cs);
+    }
     return kOk;
 }
 

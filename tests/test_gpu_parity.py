@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from decdec_amd import ext, formats as F
+from decdec_amd import _lib, ext, formats as F
 from oracle import decdec_oracle as O
 from tests.helpers import TORCH_DT, make_dec_layer, np_of, rel_err
 
@@ -128,6 +128,29 @@ def test_anyprec_gemv_bits_and_dequant(bits, dt, c_oracle):
     want_w = O.anyprec_dequant(qweight.numpy(), np_of(lut), bits)
     assert np.array_equal(np_of(w), want_w), "dequantised weights must be bit-exact LUT entries"
     want = c_oracle.anyprec_gemv(np_of(x), qweight.numpy(), np_of(lut), bits, dt)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dt == "fp16" else TOL_BF16), (mre, mae)
+
+
+@pytest.mark.parametrize("cs", [2, 4, 8])
+@pytest.mark.parametrize("K,N,dt", [(4096, 4096, "fp16"), (2048, 130, "fp16"), (1024, 64, "bf16"), (14336, 257, "fp16")])
+def test_anyprec3_tile_decoder(K, N, dt, cs, c_oracle):
+    """The optional 3-bit tile decoder (lane = row, LDS-transposed tiles, activations in SGPRs) gives the
+    same result as the oracle; N not a multiple of 64 exercises the clamped rows and the odd tail."""
+    dtype = TORCH_DT[dt]
+    g = torch.Generator().manual_seed(K * 7 + N)
+    idx = torch.randint(0, 8, (N, K), generator=g, dtype=torch.int64)
+    lut = (torch.randn(N, 8, generator=g) * 0.02).to(dtype)
+    qweight = F.pack_anyprec(idx, 3)
+    x = F.make_activation(K, g, dtype=dtype)
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    _lib.set_option("anyprec_tile", cs)
+    try:
+        ext.anyprec_gemv(x.cuda(), out, qweight.cuda(), lut.cuda(), 3)
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_option("anyprec_tile", 0)
+    want = c_oracle.anyprec_gemv(np_of(x), qweight.numpy(), np_of(lut), 3, dt)
     mre, mae = rel_err(np_of(out).reshape(-1), want)
     assert mre <= (TOL if dt == "fp16" else TOL_BF16), (mre, mae)
 
