@@ -29,6 +29,9 @@ template <> struct Elem<kFP32> {
     using store_t = float;
     static constexpr int bytes = 4;
     static __device__ __forceinline__ float load(const void* p, size_t i) { return ((const float*)p)[i]; }
+    // storage bits of element i, and their value (lets a caller request a value long before it converts it)
+    static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint32_t*)p)[i]; }
+    static __device__ __forceinline__ float from_raw(uint32_t r) { return __uint_as_float(r); }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((float*)p)[i] = v; }
     // Atomically add (v0, v1) to out[i], out[i+1]; i is even.
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
@@ -68,6 +71,10 @@ template <> struct Elem<kFP16> {
     using store_t = _Float16;
     static constexpr int bytes = 2;
     static __device__ __forceinline__ float load(const void* p, size_t i) { return (float)((const _Float16*)p)[i]; }
+    static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint16_t*)p)[i]; }
+    static __device__ __forceinline__ float from_raw(uint32_t r) {
+        const uint16_t h = (uint16_t)r; _Float16 v; __builtin_memcpy(&v, &h, 2); return (float)v;
+    }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
         half2_t v = {(_Float16)v0, (_Float16)v1};
@@ -85,6 +92,8 @@ template <> struct Elem<kBF16> {
     using store_t = uint16_t;
     static constexpr int bytes = 2;
     static __device__ __forceinline__ float load(const void* p, size_t i) { return bf16_bits_to_f32(((const uint16_t*)p)[i]); }
+    static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint16_t*)p)[i]; }
+    static __device__ __forceinline__ float from_raw(uint32_t r) { return bf16_bits_to_f32((uint16_t)r); }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
         short2_t v = {(short)f32_to_bf16_bits(v0), (short)f32_to_bf16_bits(v1)};

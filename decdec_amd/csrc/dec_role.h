@@ -318,14 +318,15 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
         float act_sum = 0.f;
         // the scales this thread needs in the merge step, requested before the row fetch so that their
         // latency hides behind it: merge task t -> word (t & 63) of segment t >> 8, output pair (t >> 6) & 3
-        float sc0[kMergeTasks], sc1[kMergeTasks];
+        // (storage bits only: a conversion here would make the thread wait for them before the first row)
+        uint32_t sc0[kMergeTasks], sc1[kMergeTasks];
 #pragma unroll
         for (int q = 0; q < kMergeTasks; ++q) {
             const uint32_t t = tid + (uint32_t)q * kDecThreads;
             const uint32_t m = (sb0 + (t >> 8)) * kWave + (t & 63u), jp = (t >> 6) & 3u;
-            const bool ok = (t < SB * 256u) && (m < p.M);
-            sc0[q] = ok ? E::load(p.scales, (size_t)(2 * jp) * p.M + m) : 0.f;
-            sc1[q] = ok ? E::load(p.scales, (size_t)(2 * jp + 1) * p.M + m) : 0.f;
+            const uint32_t mc = ((t < SB * 256u) && (m < p.M)) ? m : 0u;     // unconditional loads, clamped index
+            sc0[q] = E::load_raw(p.scales, (size_t)(2 * jp) * p.M + mc);
+            sc1[q] = E::load_raw(p.scales, (size_t)(2 * jp + 1) * p.M + mc);
         }
 
         if (col_ok) {
@@ -334,20 +335,23 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
             for (uint32_t r = rl; r < nslots; r += RL * U) {
                 uint32_t data[U];
                 float act[U];
+                int32_t row[U];
+                // all list entries first (one LDS round trip), then the requests
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const uint32_t rr = r + (uint32_t)u * RL;
-                    int32_t row = -1;
-                    float a = 0.f;
-                    if (rr < nslots) { row = lrows[rr]; a = lacts[rr]; }
-                    row = __builtin_amdgcn_readfirstlane(row);      // wave-uniform by construction
-                    if (row >= 0) {
-                        data[u] = base[(size_t)row * p.M];
-                        act[u] = a;
-                    } else {
-                        data[u] = 0x88888888u;                      // nibble 8 == value 0
-                        act[u] = 0.f;
-                    }
+                    const bool valid = rr < nslots;
+                    const uint32_t ri = valid ? rr : 0u;
+                    const int32_t rw = lrows[ri];
+                    const float a = lacts[ri];
+                    row[u] = valid ? rw : -1;
+                    act[u] = (valid && rw >= 0) ? a : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int32_t rw = __builtin_amdgcn_readfirstlane(row[u]);   // wave-uniform by construction
+                    if (rw >= 0) data[u] = base[(size_t)rw * p.M];
+                    else data[u] = 0x88888888u;                                  // nibble 8 == value 0
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -375,7 +379,9 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
                 v0 += red[(wv * 8 + 2 * jp) * kWave + lw];
                 v1 += red[(wv * 8 + 2 * jp + 1) * kWave + lw];
             }
-            E::atomic_add2(p.out, (size_t)8 * m + 2 * jp, v0 * sc0[q], v1 * sc1[q]);
+            uint32_t r0 = sc0[q], r1 = sc1[q];
+            asm volatile("" : "+v"(r0), "+v"(r1));        // first use of the scales: here, not earlier
+            E::atomic_add2(p.out, (size_t)8 * m + 2 * jp, v0 * E::from_raw(r0), v1 * E::from_raw(r1));
         }
         dec_stamp(p, bid, 3);
         __syncthreads();                                 // red is reused by the next batch
