@@ -148,10 +148,20 @@ __device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) {
     return u == 0 ? 15u : u == 1 ? 18u : u == 2 ? 21u : u == 3 ? 23u : u == 4 ? 25u : u == 5 ? 27u : u == 6 ? 29u : 31u;
 }
 
+// The four activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
+// costs a branch and a full wait each).
+// Storage bits only: converting at once would make the lane wait for the loads where they are issued.
+template <int DT>
+__device__ __forceinline__ void dec_load_x4(const DecParams& p, uint32_t lo, uint32_t len, uint32_t ch0, uint32_t (&xr)[4]) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) xr[s] = Elem<DT>::load_raw(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
+}
+
 template <int DT>
 __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
                                                  int32_t* lrows, float* lacts, uint32_t* cnt,
-                                                 uint32_t* pre, float* red, bool write_global) {
+                                                 uint32_t* pre, float* red, bool write_global,
+                                                 bool have_xpre, const uint32_t (&xpre)[4]) {
     using E = Elem<DT>;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -171,9 +181,16 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     float xv[4], a[4];
     const uint32_t ch0 = 4u * tid;
     if (scanner) {
-        // unconditional loads from clamped indices (a predicated load costs a branch and a full wait each)
+        uint32_t xr[4];
+        if (have_xpre) {                                   // uniform: requested when the workgroup started
 #pragma unroll
-        for (int s = 0; s < 4; ++s) xv[s] = E::load(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
+            for (int s = 0; s < 4; ++s) xr[s] = xpre[s];
+        } else {
+            dec_load_x4<DT>(p, lo, len, ch0, xr);
+        }
+        asm volatile("" : "+v"(xr[0]), "+v"(xr[1]), "+v"(xr[2]), "+v"(xr[3]));   // first use: here
+#pragma unroll
+        for (int s = 0; s < 4; ++s) xv[s] = E::from_raw(xr[s]);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const bool in = ch0 + s < len;
@@ -401,13 +418,22 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
     float* red = (float*)(pre + 512);
 
     dec_stamp(p, bid, 0);
+    // the scanning waves ask for the activations of the workgroup's first chunk before anything else: their
+    // latency is the head of the critical path
+    uint32_t xpre[4] = {0u, 0u, 0u, 0u};
+    const bool have_xpre = p.fused_select && p.monotone && cgid < p.num_chunks;      // uniform
+    if (have_xpre && tid < (uint32_t)kSelWaves * kWave) {
+        const uint32_t lo = cgid * kChunk;
+        const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
+        dec_load_x4<DT>(p, lo, len, 4u * tid, xpre);
+    }
     for (uint32_t i = tid; i < p.slots_per_block; i += kDecThreads) lrows[i] = -1;
     uint32_t nslots = 0;
     if (p.fused_select) {
         uint32_t t = 0;
         for (uint32_t c = cgid; c < p.num_chunks; c += p.cg, ++t) {
             __syncthreads();      // list initialised; cnt/pre of the previous chunk no longer read
-            dec_select_chunk<DT>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0);
+            dec_select_chunk<DT>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0, have_xpre && t == 0, xpre);
         }
         nslots = t * p.k_chunk;
     } else {
