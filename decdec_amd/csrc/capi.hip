@@ -404,16 +404,19 @@ int plan_sqllm(const void* input, void* output, const void* mat, const void* lut
     memset(&p, 0, sizeof(p));
     p.x = input; p.mat = (const uint32_t*)mat; p.lut = lut; p.out = output;
     p.N = N; p.K = K; p.bits = (uint32_t)bits;
-    p.nthreads = 256;
-    p.n_tiles = cdiv(N, p.nthreads);
-    uint32_t kt = g_opt.sqllm_ktiles > 0 ? (uint32_t)g_opt.sqllm_ktiles : cdiv(2048, p.n_tiles);
-    // every K range costs one rounding of the 16-bit output (one atomic add), so the split stays small
-    kt = std::max(1u, std::min(std::min(kt, 8u), K / 128 ? K / 128 : 1u));
-    p.kspan = cdiv(cdiv(K, kt), 32) * 32;
-    p.k_tiles = cdiv(K, p.kspan);
+    DD_CHECK(((uintptr_t)input % 4) == 0, "input must be 4-byte aligned");
+    // 16 waves per workgroup share 64 columns and split the workgroup's K range; the K ranges (one atomic
+    // add, i.e. one rounding of a 16-bit output, each) are few: enough for about 8 waves per SIMD, at most 8
+    const uint32_t waves = 16;
+    p.n_tiles = cdiv(N, 64);
+    uint32_t kt = g_opt.sqllm_ktiles > 0 ? (uint32_t)g_opt.sqllm_ktiles : cdiv(8192, p.n_tiles * waves);
+    kt = std::max(1u, std::min(std::min(kt, 8u), std::max(1u, K / (32u * waves))));
+    p.kslice = cdiv(cdiv(K, kt * waves), 32) * 32;
+    p.k_tiles = cdiv(K, p.kslice * waves);
     pl->d.grid = p.n_tiles * p.k_tiles;
-    pl->d.block = fused_block ? 1024u : p.nthreads;
-    pl->d.lds = sqllm_lds_bytes(p.nthreads, p.bits, p.kspan);
+    pl->d.block = 64u * waves;
+    pl->d.lds = sqllm_lds_bytes(p.bits, waves);
+    (void)fused_block;
     return kOk;
 }
 

@@ -4,15 +4,19 @@
 // 32u..32u+31 form a 96-bit little-endian stream over words 3u..3u+2, field at bit 3 (c % 32)
 // (reference decdec_extension/sqllm.cu:28-169).
 //
-// A thread owns one output column, so the packed words of 64 neighbouring columns form one coalesced
-// 256-byte wave load per matrix row.  The column's LUT sits in LDS as lut_s[value][thread] (fp32): a
-// lookup hits bank (thread % 32) whatever the value, i.e. it is conflict-free.  The activations of
-// the workgroup's K range are staged in LDS once and read as broadcasts.  fp32 accumulation; one
-// atomic add per output per K range.
+// A lane owns one output column, so the packed words of 64 neighbouring columns form one coalesced
+// 256-byte wave load per matrix row.  All waves of a workgroup work on the SAME 64 columns and split the
+// workgroup's K range between them: the columns' LUTs are converted to fp32 once per workgroup and sit in
+// LDS as lut_s[value][lane] (a lookup hits bank lane % 32 whatever the value: conflict-free), the
+// activations of a wave's channels are the same for all its lanes and therefore arrive through the
+// scalar cache and stay in SGPRs, the waves' partial sums are added in LDS, and an output receives one
+// atomic add per workgroup (k_tiles per output in all).  fp32 accumulation.
 #pragma once
 #include "common.h"
 
 namespace decdec {
+
+#define DD_SCALAR_AS __attribute__((address_space(4)))
 
 struct SqllmParams {
     const void* x;
@@ -20,83 +24,131 @@ struct SqllmParams {
     const void* lut;
     void* out;
     uint32_t N, K, bits;
-    uint32_t kspan;            // channels per workgroup along K (multiple of 32)
-    uint32_t nthreads;         // threads (= columns) that work per workgroup: multiple of 64, <= blockDim
-    uint32_t n_tiles, k_tiles;
+    uint32_t kslice;           // channels per wave (multiple of 32)
+    uint32_t n_tiles, k_tiles; // column groups of 64 x K ranges of (waves per workgroup) * kslice
 };
 
-__host__ __device__ inline size_t sqllm_lds_bytes(uint32_t nthreads, uint32_t bits, uint32_t kspan) {
-    return ((size_t)(1u << bits) * nthreads + kspan) * 4;
+__host__ __device__ inline size_t sqllm_lds_bytes(uint32_t bits, uint32_t waves) {
+    return ((size_t)(1u << bits) * 64 + (size_t)waves * 64) * 4;
 }
+
+// The 32 activations of channels c0 .. c0+31 as fp32 SGPR values: raw storage comes through the scalar
+// cache (the address is wave-uniform), element e is converted where it is used.
+template <int DT> struct SqllmX;
+template <> struct SqllmX<kFP32> {
+    uint32_t d[32];
+    __device__ __forceinline__ void load(const void* x, uint32_t c0) {
+        const DD_SCALAR_AS uint32_t* s = (const DD_SCALAR_AS uint32_t*)x + c0;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) d[i] = s[i];
+    }
+    __device__ __forceinline__ float fma(int e, float w, float acc) const { return __builtin_fmaf(w, __uint_as_float(d[e]), acc); }
+};
+template <> struct SqllmX<kFP16> {
+    uint32_t d[16];
+    __device__ __forceinline__ void load(const void* x, uint32_t c0) {
+        const DD_SCALAR_AS uint32_t* s = (const DD_SCALAR_AS uint32_t*)x + (c0 >> 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) d[i] = s[i];
+    }
+    __device__ __forceinline__ float fma(int e, float w, float acc) const {
+        const half2_t h = *(const half2_t*)&d[e >> 1];
+        return __builtin_fmaf(w, (float)h[e & 1], acc);       // mixed-precision fma, the half comes from an SGPR
+    }
+};
+template <> struct SqllmX<kBF16> {
+    uint32_t d[16];
+    __device__ __forceinline__ void load(const void* x, uint32_t c0) {
+        const DD_SCALAR_AS uint32_t* s = (const DD_SCALAR_AS uint32_t*)x + (c0 >> 1);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) d[i] = s[i];
+    }
+    __device__ __forceinline__ float fma(int e, float w, float acc) const {
+        const uint32_t b = (e & 1) ? (d[e >> 1] & 0xFFFF0000u) : (d[e >> 1] << 16);
+        return __builtin_fmaf(w, __uint_as_float(b), acc);
+    }
+};
 
 template <int DT>
 __device__ __forceinline__ void sqllm_role(const SqllmParams& p, uint32_t bid, unsigned char* smem) {
     using E = Elem<DT>;
-    const uint32_t tid = threadIdx.x, nthreads = p.nthreads;
-    if (tid >= nthreads) return;                    // surplus waves of a wider launch leave at once
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, nthreads = blockDim.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = nthreads >> 6;
     const uint32_t nt = bid % p.n_tiles, ktile = bid / p.n_tiles;
     const uint32_t L = 1u << p.bits;
-    float* lut_s = (float*)smem;                    // [L][nthreads]
-    float* xs = lut_s + (size_t)L * nthreads;       // [kspan]
-    const uint32_t n = nt * nthreads + tid;
-    const uint32_t k0 = ktile * p.kspan;
-    const uint32_t k1 = (k0 + p.kspan) < p.K ? (k0 + p.kspan) : p.K;
+    float* lut_s = (float*)smem;                    // [L][64]
+    float* part = lut_s + (size_t)L * 64;           // [nwaves][64]
+    const uint32_t n0 = nt * 64u, n = n0 + lane;
     const bool col_ok = n < p.N;
+    const uint32_t nc = col_ok ? n : p.N - 1u;      // columns past the end re-read the last one
 
-    if (col_ok)
-        for (uint32_t v = 0; v < L; ++v) lut_s[v * nthreads + tid] = E::load(p.lut, (size_t)n * L + v);
-    for (uint32_t c = k0 + tid; c < k1; c += nthreads) xs[c - k0] = E::load(p.x, c);
+    // the 64 columns' LUTs: entry idx = col * L + value, coalesced in memory
+    for (uint32_t idx = tid; idx < 64u * L; idx += nthreads) {
+        const uint32_t col = idx >> p.bits, v = idx & (L - 1u);
+        const uint32_t cn = (n0 + col < p.N) ? n0 + col : p.N - 1u;
+        lut_s[v * 64u + col] = E::load(p.lut, (size_t)cn * L + v);
+    }
+    const uint32_t k0 = (ktile * nwaves + wave) * p.kslice;
+    const uint32_t k1 = (k0 + p.kslice) < p.K ? (k0 + p.kslice) : p.K;    // may be <= k0: nothing to do
     __syncthreads();
 
     float acc = 0.f;
-    const float* lt = lut_s + tid;
-    if (!col_ok) {
-        // nothing to accumulate; stay for the lane pairing below
-    } else if (p.bits == 4) {
-        const uint32_t r0 = k0 / 8u, r1 = k1 / 8u;
-        constexpr int U = 8;
-        for (uint32_t r = r0; r < r1; r += U) {
-            uint32_t w[U];
+    const unsigned char* lt = (const unsigned char*)(lut_s + lane);       // + value * 256 bytes
+    const uint32_t* col = p.mat + nc;
+    if (p.bits == 4) {
+        uint32_t m = 0xF00u;
+        asm volatile("" : "+v"(m));                 // mask in a VGPR: all-VGPR operations issue at twice the rate
+#pragma unroll 1
+        for (uint32_t c = k0; c < k1; c += 32u) {
+            uint32_t w[4];
 #pragma unroll
-            for (int u = 0; u < U; ++u) w[u] = (r + u < r1) ? p.mat[(size_t)(r + u) * p.N + n] : 0u;
+            for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(c / 8u + u) * p.N);
+            SqllmX<DT> xs;
+            xs.load(p.x, c);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (r + u >= r1) break;
-                const float* xv = xs + (size_t)(r + u - r0) * 8;
+            for (int u = 0; u < 4; ++u) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc += lt[((w[u] >> (4 * j)) & 0xFu) * nthreads] * xv[j];
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t sh = (4 * j >= 8) ? (w[u] >> (4 * j - 8)) : (w[u] << (8 - 4 * j));
+                    const float wv = *(const float*)(lt + (sh & m));
+                    acc = xs.fma(8 * u + j, wv, acc);
+                }
             }
         }
     } else {
-        const uint32_t u0 = k0 / 32u, u1 = k1 / 32u;
-        constexpr int U = 2;
-        for (uint32_t g = u0; g < u1; g += U) {
-            uint32_t w[U][3];
+        uint32_t m = 0x700u;
+        asm volatile("" : "+v"(m));
+#pragma unroll 1
+        for (uint32_t c = k0; c < k1; c += 32u) {
+            uint32_t w[3];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
+            for (int u = 0; u < 3; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(3u * (c / 32u) + u) * p.N);
+            SqllmX<DT> xs;
+            xs.load(p.x, c);
+            // field j sits at bit 3j of the 96-bit stream w[2]:w[1]:w[0]; fields 10 and 21 straddle words
 #pragma unroll
-                for (int q = 0; q < 3; ++q)
-                    w[u][q] = (g + u < u1) ? p.mat[(size_t)(3 * (g + u) + q) * p.N + n] : 0u;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (g + u >= u1) break;
-                const float* xv = xs + (size_t)(g + u - u0) * 32;
-                const unsigned long long lo = (unsigned long long)w[u][0] | ((unsigned long long)w[u][1] << 32);
-                const unsigned long long hi = (unsigned long long)(w[u][1] >> 31) | ((unsigned long long)w[u][2] << 1);
-                // fields 0..20 live in bits 0..62 of lo; fields 21..31 in bits 63..95 = bits 0..32 of hi
-#pragma unroll
-                for (int j = 0; j < 21; ++j) acc += lt[(uint32_t)((lo >> (3 * j)) & 7ull) * nthreads] * xv[j];
-#pragma unroll
-                for (int j = 21; j < 32; ++j) acc += lt[(uint32_t)((hi >> (3 * j - 63)) & 7ull) * nthreads] * xv[j];
+            for (int j = 0; j < 32; ++j) {
+                const int bit = 3 * j, wi = bit >> 5, off = bit & 31;
+                uint32_t v;                          // (field << 8) plus bits outside the mask
+                if (off <= 29) {
+                    v = (off >= 8) ? (w[wi] >> (off - 8)) : (w[wi] << (8 - off));
+                } else {
+                    const uint32_t f = __builtin_amdgcn_alignbit(w[wi + 1], w[wi], off);   // stream >> bit, low 32 bits
+                    v = f << 8;
+                }
+                const float wv = *(const float*)(lt + (v & m));
+                acc = xs.fma(j, wv, acc);
             }
         }
     }
-    // Columns n and n+1 sit in neighbouring lanes (tile origins are even): the even lane merges both
-    // with one packed atomic.
-    const float other = __shfl_down(acc, 1, 64);
-    if (col_ok && (tid & 1u) == 0u) {
-        if (n + 1 < p.N) E::atomic_add2(p.out, n, acc, other);
-        else E::atomic_add1(p.out, n, acc);
+    part[wave * 64u + lane] = acc;
+    __syncthreads();
+    // columns n and n+1 sit in neighbouring lanes (tile origins are even): one packed atomic per pair
+    if (wave == 0 && (lane & 1u) == 0u && col_ok) {
+        float v0 = 0.f, v1 = 0.f;
+        for (uint32_t w = 0; w < nwaves; ++w) { v0 += part[w * 64u + lane]; v1 += part[w * 64u + lane + 1u]; }
+        if (n + 1u < p.N) E::atomic_add2(p.out, n, v0, v1);
+        else E::atomic_add1(p.out, n, v0);
     }
 }
 
