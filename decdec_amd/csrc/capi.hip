@@ -49,7 +49,7 @@ struct Options {
     int fusion = 1;
     int host_noncoherent = 0;
     int anyprec_rpw = 0;
-    int lutgemm_npb = 0;
+    int lutgemm_ktiles = 0;
     int sqllm_ktiles = 0;
     int dec_trace = 0;
     int anyprec_rg = 0;
@@ -65,7 +65,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "fusion")) return &g_opt.fusion;
     if (!strcmp(name, "host_noncoherent")) return &g_opt.host_noncoherent;
     if (!strcmp(name, "anyprec_rpw")) return &g_opt.anyprec_rpw;
-    if (!strcmp(name, "lutgemm_npb")) return &g_opt.lutgemm_npb;
+    if (!strcmp(name, "lutgemm_ktiles")) return &g_opt.lutgemm_ktiles;
     if (!strcmp(name, "sqllm_ktiles")) return &g_opt.sqllm_ktiles;
     if (!strcmp(name, "dec_trace")) return &g_opt.dec_trace;
     if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
@@ -350,7 +350,8 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     const bool tile_able = bits == 3 && K % 1024 == 0 && ((uintptr_t)qweight % 16) == 0 &&
                            ((uintptr_t)input % 4) == 0 && g_opt.anyprec_tile != 0;
     if (tile_able) {
-        const uint32_t cs = (g_opt.anyprec_tile == 2 || g_opt.anyprec_tile == 4) ? (uint32_t)g_opt.anyprec_tile : 8u;
+        uint32_t cs = (g_opt.anyprec_tile == 2 || g_opt.anyprec_tile == 4) ? (uint32_t)g_opt.anyprec_tile : 8u;
+        while (cs < 8u && p.W / (4u * cs) > 16u) cs *= 2u;   // at most 16 atomic adds (roundings) per 16-bit output
         p.tile_cs = cs;
         p.tile_kt = p.W / (4u * cs);
         p.tiles = cdiv(N, 64) * p.tile_kt;
@@ -377,17 +378,18 @@ int plan_lutgemm(const void* input, void* output, const void* qw, const void* al
     memset(&p, 0, sizeof(p));
     p.x = input; p.qw = (const uint32_t*)qw; p.alpha = alpha; p.q_bias = q_bias; p.out = output;
     p.N = N; p.K = K; p.bits = (uint32_t)bits; p.group_size = (uint32_t)group_size;
-    p.ktb = std::min((uint32_t)kLutgemmMaxKtb, K / 32);
-    p.k_tiles = cdiv(K / 32, p.ktb);
-    const uint32_t threads = fused_block ? 1024u : 256u;
-    uint32_t npb = g_opt.lutgemm_npb > 0 ? (uint32_t)g_opt.lutgemm_npb : (fused_block ? 2048u : 1024u);
-    npb = std::max(2u * threads, npb);               // at least one output pair per thread
-    npb += npb & 1u;
-    p.npb = npb;
-    p.n_tiles = cdiv(N, npb);
+    // 16 waves per workgroup share 64 columns and split the workgroup's K range in slices of 1..4 tiles
+    // (tables of 4 tiles per wave = 32 KB of LDS); enough K ranges for about 8 waves per SIMD
+    const uint32_t waves = 16, tiles = K / 32;
+    p.n_tiles = cdiv(N, 64);
+    uint32_t kt = g_opt.lutgemm_ktiles > 0 ? (uint32_t)g_opt.lutgemm_ktiles : cdiv(8192, p.n_tiles * waves);
+    kt = std::max(1u, kt);
+    p.slice_tiles = std::max(1u, std::min(4u, cdiv(tiles, kt * waves)));
+    p.k_tiles = cdiv(tiles, p.slice_tiles * waves);
     pl->d.grid = p.n_tiles * p.k_tiles;
-    pl->d.block = threads;
-    pl->d.lds = lutgemm_lds_bytes(p.ktb);
+    pl->d.block = 64u * waves;
+    pl->d.lds = lutgemm_lds_bytes(p.slice_tiles, waves);
+    (void)fused_block;
     return kOk;
 }
 

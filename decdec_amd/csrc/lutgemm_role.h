@@ -4,12 +4,15 @@
 // with s_b(n, c) = bit (c % 32) of q_weight[c / 32][b][n]  (reference
 // decdec_extension/lutgemm.cu:25-150; packing llm-awq/quantize/qmodule.py:61-92).
 //
-// A workgroup owns KTB consecutive 32-channel tiles and a range of outputs.  It first builds, from
-// the activations alone, the 256-entry signed subset-sum table of every 8-channel group of its tiles
-// in LDS (fp32, so table entries carry no rounding), then every thread walks two adjacent outputs:
-// one coalesced 8-byte load per (tile, bit plane), four table lookups per 32-bit word.  Partial sums
-// stay in fp32 registers across all tiles of the workgroup, so an output receives K / (32 KTB) atomic
-// adds instead of the reference's K / 32.
+// A lane owns one output column (the packed words of 64 neighbouring columns are one coalesced 256-byte
+// wave load); the waves of a workgroup work on the same 64 columns and split the workgroup's K range.
+// The signed sums depend on the activations only, so the workgroup first builds, for every group of FOUR
+// channels of its K range, the 16-entry table of signed subset sums in LDS (fp32: entries carry no
+// rounding); a 32-bit word of a bit plane then costs eight lookups.  Sixteen-entry tables are 16
+// consecutive dwords, i.e. 16 different LDS banks: whatever nibbles the 64 lanes hold, a lookup is
+// conflict-free (equal nibbles are one broadcast), which 256-entry byte tables are not.  Partial sums stay
+// in fp32 registers, the waves are added in LDS, and an output receives one atomic add per workgroup
+// (k_tiles per output) instead of the reference's K / 32.
 #pragma once
 #include "common.h"
 
@@ -22,74 +25,99 @@ struct LutgemmParams {
     const void* q_bias;        // [K/group][N]
     void* out;
     uint32_t N, K, bits, group_size;
-    uint32_t ktb;              // 32-channel tiles per workgroup
-    uint32_t npb;              // outputs per workgroup (even)
-    uint32_t n_tiles, k_tiles;
+    uint32_t slice_tiles;      // 32-channel tiles per wave
+    uint32_t n_tiles, k_tiles; // column groups of 64 x K ranges of (waves per workgroup) * slice_tiles tiles
 };
 
-constexpr int kLutgemmMaxKtb = 8;
+constexpr int kLutgemmMaxBits = 8;
 
-__host__ __device__ inline size_t lutgemm_lds_bytes(uint32_t ktb) {
-    return (size_t)ktb * 4 * 256 * 4 + (size_t)ktb * 4;
+__host__ __device__ inline size_t lutgemm_lds_bytes(uint32_t slice_tiles, uint32_t waves) {
+    const size_t tiles = (size_t)slice_tiles * waves;
+    return tiles * 8 * 16 * 4 + tiles * 4 + (size_t)waves * 64 * 4;
+}
+
+// signed sum of the 32 activations of a tile selected by the bits of w: eight conflict-free lookups
+__device__ __forceinline__ float lutgemm_word(const unsigned char* tb, uint32_t w, uint32_t m) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t sh = (j == 0) ? (w << 2) : (w >> (4 * j - 2));
+        s += *(const float*)(tb + j * 64 + (sh & m));
+    }
+    return s;
 }
 
 template <int DT>
 __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bid, unsigned char* smem) {
     using E = Elem<DT>;
-    const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, nthreads = blockDim.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), nwaves = nthreads >> 6;
     const uint32_t nt = bid % p.n_tiles, ktile = bid / p.n_tiles;
-    const uint32_t kt0 = ktile * p.ktb;
-    const uint32_t total_kt = p.K / 32u;
-    const uint32_t nkt = (kt0 + p.ktb) <= total_kt ? p.ktb : (total_kt - kt0);
-    float* tab = (float*)smem;                       // [ktb][4][256]
-    float* xsum = tab + (size_t)p.ktb * 1024;        // [ktb]
+    const uint32_t total_tiles = p.K / 32u;
+    const uint32_t wg_tiles = p.slice_tiles * nwaves;
+    const uint32_t t0 = ktile * wg_tiles;                                   // first tile of the workgroup
+    const uint32_t nt_wg = (t0 + wg_tiles) <= total_tiles ? wg_tiles : (total_tiles - t0);
+    float* tab = (float*)smem;                       // [wg_tiles][8][16]
+    float* xsum = tab + (size_t)wg_tiles * 128;      // [wg_tiles]
+    float* part = xsum + wg_tiles;                   // [nwaves][64]
 
-    // subset-sum tables: tab[kt][y][pat] = sum_j (bit j of pat ? +1 : -1) * x[32 (kt0+kt) + 8 y + j]
-    for (uint32_t idx = tid; idx < nkt * 1024u; idx += nthreads) {
-        const uint32_t pat = idx & 255u, grp = idx >> 8;            // grp = kt*4 + y
-        const size_t c0 = (size_t)32 * kt0 + (size_t)8 * grp;
-        float s = 0.f;
+    // tables: tab[(tile * 8 + j) * 16 + pat] = sum_i (bit i of pat ? +1 : -1) * x[32 tile + 4 j + i]
+    for (uint32_t T = tid; T < nt_wg * 8u; T += nthreads) {
+        const size_t c0 = (size_t)32 * t0 + (size_t)4 * T;
+        const float x0 = E::load(p.x, c0), x1 = E::load(p.x, c0 + 1), x2 = E::load(p.x, c0 + 2), x3 = E::load(p.x, c0 + 3);
+        const float lo[4] = {-x0 - x1, x0 - x1, -x0 + x1, x0 + x1};
+        const float hi[4] = {-x2 - x3, x2 - x3, -x2 + x3, x2 + x3};
+        float* dst = tab + (size_t)T * 16;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float xv = E::load(p.x, c0 + j);
-            s += ((pat >> j) & 1u) ? xv : -xv;
-        }
-        tab[idx] = s;
+        for (int q = 0; q < 16; ++q) dst[q] = lo[q & 3] + hi[q >> 2];
     }
     __syncthreads();
-    if (tid < nkt) xsum[tid] = tab[tid * 1024 + 255] + tab[tid * 1024 + 511] + tab[tid * 1024 + 767] + tab[tid * 1024 + 1023];
+    for (uint32_t t = tid; t < nt_wg; t += nthreads) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += tab[(size_t)(t * 8 + j) * 16 + 15];
+        xsum[t] = s;
+    }
     __syncthreads();
 
-    const uint32_t n_begin = nt * p.npb;
-    const uint32_t n_end = (n_begin + p.npb) < p.N ? (n_begin + p.npb) : p.N;
-    for (uint32_t n = n_begin + 2 * tid; n < n_end; n += 2 * nthreads) {
-        const bool pair = (n + 1 < n_end) && ((p.N & 1u) == 0u);   // 8-byte aligned pair load
-        float acc0 = 0.f, acc1 = 0.f;
-        for (uint32_t kt = 0; kt < nkt; ++kt) {
-            const uint32_t g = (32u * (kt0 + kt)) / p.group_size;
-            const float* t = tab + (size_t)kt * 1024;
-            const float xs = xsum[kt];
-            acc0 += E::load(p.q_bias, (size_t)g * p.N + n) * xs;
-            if (n + 1 < n_end) acc1 += E::load(p.q_bias, (size_t)g * p.N + n + 1) * xs;
-            for (uint32_t b = 0; b < p.bits; ++b) {
-                const size_t wo = ((size_t)(kt0 + kt) * p.bits + b) * p.N + n;
-                uint32_t w0, w1 = 0u;
-                if (pair) { const u32x2 w = *(const u32x2*)(p.qw + wo); w0 = w[0]; w1 = w[1]; }
-                else { w0 = p.qw[wo]; if (n + 1 < n_end) w1 = p.qw[wo + 1]; }
-                const size_t ao = ((size_t)g * p.bits + b) * p.N + n;
-                const float t0 = t[w0 & 255u] + t[256 + ((w0 >> 8) & 255u)] + t[512 + ((w0 >> 16) & 255u)] + t[768 + (w0 >> 24)];
-                acc0 += E::load(p.alpha, ao) * t0;
-                if (n + 1 < n_end) {
-                    const float t1 = t[w1 & 255u] + t[256 + ((w1 >> 8) & 255u)] + t[512 + ((w1 >> 16) & 255u)] + t[768 + (w1 >> 24)];
-                    acc1 += E::load(p.alpha, ao + 1) * t1;
-                }
+    const uint32_t n0 = nt * 64u, n = n0 + lane;
+    const bool col_ok = n < p.N;
+    const uint32_t nc = col_ok ? n : p.N - 1u;       // columns past the end re-read the last one
+    const uint32_t lt0 = wave * p.slice_tiles;       // local tiles of this wave: [lt0, lt1)
+    const uint32_t lt1 = (lt0 + p.slice_tiles) < nt_wg ? (lt0 + p.slice_tiles) : nt_wg;
+    uint32_t m = 0x3Cu;
+    asm volatile("" : "+v"(m));                      // mask in a VGPR: all-VGPR operations issue at twice the rate
+    float acc = 0.f;
+#pragma unroll 1
+    for (uint32_t lt = lt0; lt < lt1; ++lt) {
+        const uint32_t gt = t0 + lt;                 // global tile
+        const uint32_t g = (32u * gt) / p.group_size;
+        uint32_t w[kLutgemmMaxBits];
+        uint32_t araw[kLutgemmMaxBits];
+        // every request of the tile first, then the lookups
+#pragma unroll
+        for (int b = 0; b < kLutgemmMaxBits; ++b) {
+            if ((uint32_t)b < p.bits) {
+                w[b] = __builtin_nontemporal_load(p.qw + ((size_t)gt * p.bits + b) * p.N + nc);
+                araw[b] = E::load_raw(p.alpha, ((size_t)g * p.bits + b) * p.N + nc);
             }
         }
-        if ((n + 1 < n_end) && ((n & 1u) == 0u)) E::atomic_add2(p.out, n, acc0, acc1);
-        else {
-            E::atomic_add1(p.out, n, acc0);
-            if (n + 1 < n_end) E::atomic_add1(p.out, n + 1, acc1);
+        const uint32_t braw = E::load_raw(p.q_bias, (size_t)g * p.N + nc);
+        const unsigned char* tb = (const unsigned char*)(tab + (size_t)lt * 128);
+        acc += E::from_raw(braw) * xsum[lt];
+#pragma unroll
+        for (int b = 0; b < kLutgemmMaxBits; ++b) {
+            if ((uint32_t)b < p.bits) acc += E::from_raw(araw[b]) * lutgemm_word(tb, w[b], m);
         }
+    }
+    part[wave * 64u + lane] = acc;
+    __syncthreads();
+    // columns n and n+1 sit in neighbouring lanes (tile origins are even): one packed atomic per pair
+    if (wave == 0 && (lane & 1u) == 0u && col_ok) {
+        float v0 = 0.f, v1 = 0.f;
+        for (uint32_t w2 = 0; w2 < nwaves; ++w2) { v0 += part[w2 * 64u + lane]; v1 += part[w2 * 64u + lane + 1u]; }
+        if (n + 1u < p.N) E::atomic_add2(p.out, n, v0, v1);
+        else E::atomic_add1(p.out, n, v0);
     }
 }
 

@@ -54,7 +54,7 @@ int decdec_version(void);
 
 /* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
  * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
- * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "lutgemm_npb",
+ * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "lutgemm_ktiles",
  * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
