@@ -152,6 +152,106 @@ def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
             "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": MEASURED_TRAFFIC.get(name)}
 
 
+def kernels_leg(torch, ext, F):
+    """Per-kernel table at the configuration shapes: us per launch (graph replay over private weight copies),
+    algorithmic GB/s and fraction of the roofline that bounds the kernel (HBM 8000 GB/s for the base GEMVs,
+    the 64 GB/s host link for DEC), and the fused DEC + GEMV launch with its slowdown."""
+    dev = "cuda"
+    g = torch.Generator().manual_seed(1)
+
+    def graph_time(fn, reps=20, iters=20):
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            for _ in range(3):
+                fn()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=st):
+            for _ in range(reps):
+                fn()
+        for _ in range(3):
+            gr.replay()
+        torch.cuda.synchronize()
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(st):
+            a.record(st)
+            for _ in range(iters):
+                gr.replay()
+            b.record(st)
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters / reps * 1e3
+
+    def dec_cfg(K, N, kc, ntb):
+        rows = torch.zeros(K, dtype=torch.int32, device=dev)
+        acts = torch.zeros(K, dtype=torch.float16, device=dev)
+        th = F.calibrate_thresholds(K, g, draws=8)
+        cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32)
+        sc = torch.rand(N).half()
+        ctx = ext.create_dec_context(ntb, rows, acts)
+        return (rows, acts, th, ctx), ext.create_dec_config(ctx, kc, cheat, sc, th)
+
+    def randint(shape):
+        return torch.randint(-2 ** 31, 2 ** 31 - 1, shape, dtype=torch.int32, device=dev)
+
+    rows_out = []
+    cases = []
+    for K, N in [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (8192, 8192), (8192, 28672), (28672, 8192)]:
+        cases.append(("anyprec3", K, N))
+    for K, N in [(5120, 7680), (5120, 5120), (5120, 35840), (17920, 5120)]:
+        cases.append(("lutgemm3g128", K, N))
+    for K, N in [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)]:
+        cases.append(("sqllm4", K, N))
+    for kind, K, N in cases:
+        x = F.make_activation(K, g).to(dev)
+        out = torch.zeros(1, 1, N, device=dev, dtype=torch.float16)
+        if kind == "anyprec3":
+            by = 3 * K * N // 8 + N * 16 + 2 * K + 2 * N
+            nb = max(2, min(12, int(6e8 // by)))
+            ws = [randint((3, N, K // 32)) for _ in range(nb)]
+            lut = torch.randn(N, 8, device=dev, dtype=torch.float16)
+            base = lambda j: ext.anyprec_gemv(x, out, ws[j], lut, 3)
+            fused = lambda c, j: ext.dec_anyprec(c, x, out, ws[j], lut, 3)
+        elif kind == "lutgemm3g128":
+            by = (K // 32) * 3 * N * 4 + (K // 128) * 3 * N * 2 + (K // 128) * N * 2 + 2 * K + 2 * N
+            nb = max(2, min(12, int(6e8 // by)))
+            ws = [randint((K // 32, 3, N)) for _ in range(nb)]
+            alpha = torch.rand(K // 128, 3, N, device=dev).half() * 0.01
+            qb = torch.rand(K // 128, N, device=dev).half() * 0.01
+            base = lambda j: ext.lutgemm_gemv(x, out, ws[j], alpha, qb, 3, 128)
+            fused = lambda c, j: ext.dec_lutgemm(c, x, out, ws[j], alpha, qb, 3, 128)
+        else:
+            by = K * 4 // 32 * N * 4 + N * 16 * 2 + 2 * K + 2 * N
+            nb = max(2, min(12, int(6e8 // by)))
+            ws = [randint((K * 4 // 32, N)) for _ in range(nb)]
+            lut = (torch.randn(N, 16, device=dev) * 0.02).half()
+            base = lambda j: ext.sqllm_gemv(x, out, ws[j], lut, 4)
+            fused = lambda c, j: ext.dec_sqllm(c, x, out, ws[j], lut, 4)
+        i = [0]
+
+        def run_base():
+            i[0] += 1
+            base(i[0] % nb)
+        tb = graph_time(run_base)
+        keep, cfg = dec_cfg(K, N, 32, 8)
+
+        def run_fused():
+            i[0] += 1
+            fused(cfg, i[0] % nb)
+        tf = graph_time(run_fused, reps=10, iters=10)
+        td = graph_time(lambda: ext.dec(cfg, x, out), reps=10, iters=10)
+        hb = 32 * K // 1024 * N // 2
+        rows_out.append({"kernel": kind, "K": K, "N": N, "base_us": round(tb, 2), "base_gbs": round(by / tb / 1e3, 1),
+                         "base_frac_hbm": round(by / tb / 1e3 / HBM_PEAK_GBS, 3), "dec_us": round(td, 2),
+                         "dec_host_gbs": round(hb / td / 1e3, 1), "dec_frac_link": round(hb / td / 1e3 / 64.0, 3),
+                         "fused_us": round(tf, 2), "slowdown_pct": round((tf / tb - 1) * 100, 1)})
+        print(json.dumps(rows_out[-1]), file=sys.stderr, flush=True)
+        ext.destroy_dec_config(cfg)
+        ext.destroy_dec_context(keep[3])
+        del ws
+    return rows_out
+
+
 def cpu_baseline_leg(protos, budget_s=15.0):
     """The same per-layer path (select + residual rows + any-precision GEMV) in the C oracle on the host
     cores, one layer of each shape, scaled to a token (32 layers)."""
@@ -191,8 +291,9 @@ def main():
     ap.add_argument("--n-tb", type=int, default=8)
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--leg", choices=["all", "roofline"], default="all",
-                    help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter collection)")
+    ap.add_argument("--leg", choices=["all", "roofline", "kernels"], default="all",
+                    help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
+                         "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 8)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
@@ -204,6 +305,9 @@ def main():
     _lib.load()
     torch.cuda.set_device(0)
 
+    if args.leg == "kernels":
+        print(json.dumps({"kernels": kernels_leg(torch, ext, F)}))
+        return
     if args.leg == "roofline":
         _, _, protos, _ = build_layer_set(torch, F, 0, args.k_chunk, seed=0)
         print(json.dumps({"roofline": roofline_leg(torch, ext, protos, iters=48, calibrate_copy=True)}))
