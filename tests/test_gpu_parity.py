@@ -432,3 +432,49 @@ def test_full_size_layer_properties():
     assert ((r // 1024) == np.repeat(np.arange(K2 // 1024), k_chunk)).all()
     assert torch.equal(acts[:k], x[0, 0][torch.from_numpy(r).long().cuda()])
     ext.destroy_dec_config(cfg)
+
+
+def test_full_size_lutgemm_and_sqllm_against_dense_torch():
+    """Phi-3-medium gate_up (5120 -> 35840, LUT-GEMM 3-bit, group 128) and Llama-3-8B gate (4096 -> 14336,
+    SqueezeLLM 4-bit) at full size: the packed operands are expanded to a dense fp32 matrix with plain torch
+    ops on the GPU (bit extraction, gather) and multiplied; the HIP result must agree to the output tolerance."""
+    g = torch.Generator().manual_seed(3)
+    dev = "cuda"
+    # LUT-GEMM: w[c, n] = q_bias[g, n] + sum_b alpha[g, b, n] * (2 bit - 1)
+    K, N, bits, grp = 5120, 35840, 3, 128
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, bits, N), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    alpha = (torch.rand(K // grp, bits, N, generator=g) * 0.01).half().to(dev)
+    qb = ((torch.rand(K // grp, N, generator=g) - 0.5) * 0.01).half().to(dev)
+    x = F.make_activation(K, g).to(dev)
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device=dev)
+    ext.lutgemm_gemv(x, out, qw, alpha, qb, bits, grp)
+    ref = torch.zeros(N, dtype=torch.float32, device=dev)
+    xf = x.float().reshape(-1)
+    shifts = torch.arange(32, device=dev, dtype=torch.int32).view(1, 32, 1)
+    for t0 in range(0, K // 32, 16):                      # 16 tiles (512 channels) at a time
+        tiles = qw[t0:t0 + 16]                            # [16, bits, N]
+        w = torch.zeros(16, 32, N, dtype=torch.float32, device=dev)
+        gi = (torch.arange(t0, t0 + 16, device=dev) * 32) // grp
+        for b in range(bits):
+            sign = ((tiles[:, b, :].unsqueeze(1) >> shifts) & 1).float() * 2 - 1          # [16, 32, N]
+            w += alpha[gi, b, :].float().unsqueeze(1) * sign
+        w += qb[gi].float().unsqueeze(1)
+        ref += (xf[t0 * 32:(t0 + 16) * 32].view(16, 32, 1) * w).sum(dim=(0, 1))
+    torch.cuda.synchronize()
+    assert ((out.float().reshape(-1) - ref).abs().max() / ref.abs().max()) < 1e-2
+    del qw, alpha, qb, w
+    # SqueezeLLM 4-bit: channel c of column n = nibble c % 8 of mat[c // 8, n]
+    K, N = 4096, 14336
+    mat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, N), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    lut = (torch.randn(N, 16, generator=g) * 0.02).half().to(dev)
+    x = F.make_activation(K, g).to(dev)
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device=dev)
+    ext.sqllm_gemv(x, out, mat, lut, 4)
+    xf = x.float().reshape(-1)
+    ref = torch.zeros(N, dtype=torch.float32, device=dev)
+    lutT = lut.float().T.contiguous()                     # [16, N]
+    for j in range(8):
+        idx = ((mat >> (4 * j)) & 15).long()              # [K/8, N]
+        ref += (torch.gather(lutT, 0, idx) * xf[j::8].view(-1, 1)).sum(0)
+    torch.cuda.synchronize()
+    assert ((out.float().reshape(-1) - ref).abs().max() / ref.abs().max()) < 1e-2
