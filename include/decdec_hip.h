@@ -54,7 +54,7 @@ int decdec_version(void);
 
 /* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
  * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
- * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "lutgemm_ktiles",
+ * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "anyprec_tile" (3-bit LDS-transposed tile decoder, waves per tile 2/4/8, 0 = off [default]), "lutgemm_ktiles",
  * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
@@ -112,7 +112,8 @@ int decdec_lutgemm_gemv(const void* input, void* output, const void* q_weight, c
                         const void* q_bias, int bitwidth, int group_size, int dtype,
                         uint32_t in_features, uint32_t out_features, void* stream);
 /* sqllm_gemv (decdec.cu:594-603 -> VecQuant{3,4}MatMulKernelNUQPerChannel sqllm.cu:28-169).
- * qweight int32 [in*bitwidth/32, out], lut [out, 2^bitwidth]; bitwidth 3 or 4. */
+ * qweight int32 [in*bitwidth/32, out], lut [out, 2^bitwidth]; bitwidth 3 or 4.  `input` must be 4-byte
+ * aligned (it is read through the scalar cache). */
 int decdec_sqllm_gemv(const void* input, void* output, const void* qweight, const void* lut,
                       int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
                       void* stream);
