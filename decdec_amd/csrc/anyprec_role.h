@@ -174,6 +174,35 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return v;
 }
 
+// The same reduction for G values at once, written out so that every step is ONE instruction
+// (v_add_f32_dpp with destination = second source; lanes disabled by row_mask keep their value, which is
+// "add zero") and so that the steps of the G values interleave: a DPP source must not be read in the two
+// issue slots after the instruction that wrote it.
+#define DD_DPP_STEP(ctrl) \
+    "v_add_f32_dpp %0, %0, %0 " ctrl "\n v_add_f32_dpp %1, %1, %1 " ctrl "\n" \
+    "v_add_f32_dpp %2, %2, %2 " ctrl "\n v_add_f32_dpp %3, %3, %3 " ctrl "\n"
+__device__ __forceinline__ void wave_sum_dpp4(float& a, float& b, float& c, float& d) {
+    asm volatile("s_nop 1\n"
+                 DD_DPP_STEP("quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf")
+                 DD_DPP_STEP("quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf")
+                 DD_DPP_STEP("row_ror:4 row_mask:0xf bank_mask:0xf")
+                 DD_DPP_STEP("row_ror:8 row_mask:0xf bank_mask:0xf")
+                 DD_DPP_STEP("row_bcast:15 row_mask:0xa bank_mask:0xf")
+                 DD_DPP_STEP("row_bcast:31 row_mask:0xc bank_mask:0xf")
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+#undef DD_DPP_STEP
+template <int RB>
+__device__ __forceinline__ void wave_sum_rows(float (&v)[RB]) {
+    if constexpr (RB % 4 == 0) {
+#pragma unroll
+        for (int r = 0; r < RB; r += 4) wave_sum_dpp4(v[r], v[r + 1], v[r + 2], v[r + 3]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) v[r] = wave_sum_dpp(v[r]);
+    }
+}
+
 #define DD_CONST_AS __attribute__((address_space(4)))
 
 // One wave's share of the GEMV: slice `s` of RB consecutive rows.  All weight words of the RB rows are
@@ -192,8 +221,8 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
     const bool wave_active = g < p.rg;
     const uint32_t wi = (sgrp * p.S + s) * kWave + lane;    // word index inside the row
     const bool lane_ok = wi < p.W;
-    const uint32_t wi_c = lane_ok ? wi : (p.W - 1u);        // out-of-range lanes re-read a valid word and
-                                                            // multiply it with zero activations
+    const uint32_t wi_c = lane_ok ? wi : (p.W - 1u);        // out-of-range lanes re-read a valid word; their
+                                                            // sums are dropped
     const bool direct = p.S * p.sgroups <= 2u;              // few slices: every wave merges its own sums
     float* part = (float*)smem;                             // [rows_per_block][S]
     float* wlut = part + (size_t)rows_per_block * p.S + (size_t)wave * 256;
@@ -206,6 +235,7 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
         // are still streaming in.
         uint32_t xr[4][4];
         anyprec_issue_x(p, wi_c, xr);
+        const uint32_t word_off = wi_c * 4u;        // byte offset of the lane's word inside a row
         u32x4 lut4[RB];
         if constexpr (BITS == 3) {
 #pragma unroll
@@ -219,17 +249,14 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
-            const uint32_t* rp = p.qweight + (size_t)row * p.W;
+            const char* rp = (const char*)(p.qweight + (size_t)row * p.W);      // wave-uniform
 #pragma unroll
-            for (int pl = 0; pl < BITS; ++pl) q[r][pl] = __builtin_nontemporal_load(rp + pl * plane_stride + wi_c);
+            for (int pl = 0; pl < BITS; ++pl)
+                q[r][pl] = __builtin_nontemporal_load((const uint32_t*)(rp + (size_t)pl * plane_stride * 4 + word_off));
             __builtin_amdgcn_sched_barrier(0);      // keep the requests in row order: they return in issue order
         }
         uint32_t xp[8][2];
         anyprec_arrange_x(xr, xp);
-        if (!lane_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) { xp[e][0] = 0u; xp[e][1] = 0u; }
-        }
         float sums[RB];
         Anyprec3Masks mk;
         mk.init();
@@ -248,9 +275,10 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
                 __builtin_amdgcn_wave_barrier();
                 acc = anyprec_generic_word<DT, BITS>(q[r], wlut, xp, 0.f);
             }
-            sums[r] = wave_sum_dpp(acc);                    // total in lane 63
+            sums[r] = lane_ok ? acc : 0.f;                  // lanes past the row's end decoded a re-read word
             __builtin_amdgcn_sched_barrier(0);              // decode row by row, as the rows arrive
         }
+        wave_sum_rows<RB>(sums);                            // totals in lane 63
         if (lane == 63) {
             if (direct) {
 #pragma unroll

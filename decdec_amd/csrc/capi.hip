@@ -332,7 +332,7 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     const uint32_t s_total = cdiv(p.W, 64);
     p.sgroups = cdiv(s_total, 16);
     p.S = cdiv(s_total, p.sgroups);
-    p.rg = fused_block ? std::max(1u, 16u / p.S) : std::max(1u, 8u / p.S);
+    p.rg = fused_block ? std::max(1u, 16u / p.S) : std::max(1u, 4u / p.S);   // 256-thread workgroups measured best
     if (!fused_block && g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
     // Rows per wave: every wave requests all its rows at once, so more rows per wave mean more bytes
     // in flight per resident wave (large matrices), fewer rows mean more waves to share the decode
