@@ -411,13 +411,17 @@ int plan_sqllm(const void* input, void* output, const void* mat, const void* lut
     // add, i.e. one rounding of a 16-bit output, each) are few: enough for about 8 waves per SIMD, at most 8
     const uint32_t waves = 16;
     p.n_tiles = cdiv(N, 64);
-    uint32_t kt = g_opt.sqllm_ktiles > 0 ? (uint32_t)g_opt.sqllm_ktiles : cdiv(8192, p.n_tiles * waves);
+    // 16-bit types: the pair table takes 68 KB of LDS, two workgroups fit a CU, so at most 512 workgroups run
+    // at once; that many K ranges (measured best), fp32: enough for about 8 waves per SIMD
+    uint32_t kt = dtype != DECDEC_FP32 ? 512u / std::min(512u, p.n_tiles) : cdiv(8192, p.n_tiles * waves);
+    if (g_opt.sqllm_ktiles > 0) kt = (uint32_t)g_opt.sqllm_ktiles;
     kt = std::max(1u, std::min(std::min(kt, 8u), std::max(1u, K / (32u * waves))));
     p.kslice = cdiv(cdiv(K, kt * waves), 32) * 32;
     p.k_tiles = cdiv(K, p.kslice * waves);
     pl->d.grid = p.n_tiles * p.k_tiles;
     pl->d.block = 64u * waves;
-    pl->d.lds = sqllm_lds_bytes(p.bits, waves);
+    pl->d.lds = sqllm_lds_bytes(p.bits, waves, dtype != DECDEC_FP32);
+    DD_CHECK(dtype == DECDEC_FP32 || ((uintptr_t)lut % 16) == 0, "lut must be 16-byte aligned");
     (void)fused_block;
     return kOk;
 }

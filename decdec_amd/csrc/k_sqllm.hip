@@ -17,7 +17,24 @@ __global__ __launch_bounds__(1024) void dec_sqllm_kernel(const DecParams dp, con
     else sqllm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
 }
 
+// The 4-bit pair table needs more than the 64 KB of dynamic LDS a kernel gets by default.
+template <typename K>
+static hipError_t allow_large_lds(K kernel) {
+    return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+}
+static hipError_t sqllm_prepare() {
+    static hipError_t done = [] {
+        hipError_t e = hipSuccess;
+        auto acc = [&e](hipError_t r) { if (e == hipSuccess) e = r; };
+        acc(allow_large_lds(sqllm_kernel<kFP32>)); acc(allow_large_lds(sqllm_kernel<kFP16>)); acc(allow_large_lds(sqllm_kernel<kBF16>));
+        acc(allow_large_lds(dec_sqllm_kernel<kFP32>)); acc(allow_large_lds(dec_sqllm_kernel<kFP16>)); acc(allow_large_lds(dec_sqllm_kernel<kBF16>));
+        return e;
+    }();
+    return done;
+}
+
 hipError_t launch_sqllm(int dt, const SqllmParams& p, const LaunchDims& d, hipStream_t s) {
+    if (hipError_t e = sqllm_prepare(); e != hipSuccess) return e;
     switch (dt) {
         case kFP32: hipLaunchKernelGGL(sqllm_kernel<kFP32>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
         case kFP16: hipLaunchKernelGGL(sqllm_kernel<kFP16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
@@ -29,6 +46,7 @@ hipError_t launch_sqllm(int dt, const SqllmParams& p, const LaunchDims& d, hipSt
 
 hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
                               const SqllmParams& gp, const LaunchDims& d, hipStream_t s) {
+    if (hipError_t e = sqllm_prepare(); e != hipSuccess) return e;
     const dim3 grid(dec_blocks + d.grid), block(d.block);
     switch (dt) {
         case kFP32: hipLaunchKernelGGL(dec_sqllm_kernel<kFP32>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
