@@ -33,18 +33,51 @@ constexpr int kLutgemmMaxBits = 8;
 
 __host__ __device__ inline size_t lutgemm_lds_bytes(uint32_t slice_tiles, uint32_t waves) {
     const size_t tiles = (size_t)slice_tiles * waves;
-    return tiles * 8 * 16 * 4 + tiles * 4 + (size_t)waves * 64 * 4;
+    return 512 + tiles * 8 * 16 * 4 + tiles * 4 + (size_t)waves * 64 * 4;    // 512: the tables are aligned to their size
 }
 
-// signed sum of the 32 activations of a tile selected by the bits of w: eight conflict-free lookups
-__device__ __forceinline__ float lutgemm_word(const unsigned char* tb, uint32_t w, uint32_t m) {
+#define DD_LDS_AS __attribute__((address_space(3)))
+
+// signed sum of the 32 activations of a tile selected by the bits of w: eight conflict-free lookups.
+// tb = LDS byte address of the tile's tables (a multiple of 512), m = 0x3C in a VGPR; a lookup is a
+// shift, an and-or that forms the address, the read and an add.
+__device__ __forceinline__ float lutgemm_word(uint32_t tb, uint32_t w, uint32_t m) {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const uint32_t sh = (j == 0) ? (w << 2) : (w >> (4 * j - 2));
-        s += *(const float*)(tb + j * 64 + (sh & m));
+        const uint32_t addr = (sh & m) | tb;
+        s += *(const DD_LDS_AS float*)(uintptr_t)(addr + j * 64);
     }
     return s;
+}
+
+// The walk of one wave over its tiles for a compile-time number of bit planes: all requests of a tile
+// (plane words, alpha, bias) are issued before its lookups.
+template <int DT, int BITS>
+__device__ __forceinline__ float lutgemm_tiles(const LutgemmParams& p, uint32_t t0, uint32_t lt0, uint32_t lt1,
+                                               uint32_t nc, uint32_t tab_lds, const float* xsum) {
+    using E = Elem<DT>;
+    uint32_t m = 0x3Cu;
+    asm volatile("" : "+v"(m));                      // mask in a VGPR
+    float acc = 0.f;
+#pragma unroll 1
+    for (uint32_t lt = lt0; lt < lt1; ++lt) {
+        const uint32_t gt = t0 + lt;                 // global tile
+        const uint32_t g = (32u * gt) / p.group_size;
+        uint32_t w[BITS], araw[BITS];
+#pragma unroll
+        for (int b = 0; b < BITS; ++b) {
+            w[b] = __builtin_nontemporal_load(p.qw + ((size_t)gt * BITS + b) * p.N + nc);
+            araw[b] = E::load_raw(p.alpha, ((size_t)g * BITS + b) * p.N + nc);
+        }
+        const uint32_t braw = E::load_raw(p.q_bias, (size_t)g * p.N + nc);
+        const uint32_t tb = tab_lds + lt * 512u;
+        acc += E::from_raw(braw) * xsum[lt];
+#pragma unroll
+        for (int b = 0; b < BITS; ++b) acc += E::from_raw(araw[b]) * lutgemm_word(tb, w[b], m);
+    }
+    return acc;
 }
 
 template <int DT>
@@ -57,7 +90,9 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
     const uint32_t wg_tiles = p.slice_tiles * nwaves;
     const uint32_t t0 = ktile * wg_tiles;                                   // first tile of the workgroup
     const uint32_t nt_wg = (t0 + wg_tiles) <= total_tiles ? wg_tiles : (total_tiles - t0);
-    float* tab = (float*)smem;                       // [wg_tiles][8][16]
+    // tables start at a multiple of 512 bytes of LDS, so that a table address can be formed with an OR
+    const uint32_t smem_lds = (uint32_t)(uintptr_t)(DD_LDS_AS unsigned char*)smem;
+    float* tab = (float*)(smem + ((512u - (smem_lds & 511u)) & 511u));   // [wg_tiles][8][16]
     float* xsum = tab + (size_t)wg_tiles * 128;      // [wg_tiles]
     float* part = xsum + wg_tiles;                   // [nwaves][64]
 
@@ -85,30 +120,17 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
     const uint32_t nc = col_ok ? n : p.N - 1u;       // columns past the end re-read the last one
     const uint32_t lt0 = wave * p.slice_tiles;       // local tiles of this wave: [lt0, lt1)
     const uint32_t lt1 = (lt0 + p.slice_tiles) < nt_wg ? (lt0 + p.slice_tiles) : nt_wg;
-    uint32_t m = 0x3Cu;
-    asm volatile("" : "+v"(m));                      // mask in a VGPR: all-VGPR operations issue at twice the rate
-    float acc = 0.f;
-#pragma unroll 1
-    for (uint32_t lt = lt0; lt < lt1; ++lt) {
-        const uint32_t gt = t0 + lt;                 // global tile
-        const uint32_t g = (32u * gt) / p.group_size;
-        uint32_t w[kLutgemmMaxBits];
-        uint32_t araw[kLutgemmMaxBits];
-        // every request of the tile first, then the lookups
-#pragma unroll
-        for (int b = 0; b < kLutgemmMaxBits; ++b) {
-            if ((uint32_t)b < p.bits) {
-                w[b] = __builtin_nontemporal_load(p.qw + ((size_t)gt * p.bits + b) * p.N + nc);
-                araw[b] = E::load_raw(p.alpha, ((size_t)g * p.bits + b) * p.N + nc);
-            }
-        }
-        const uint32_t braw = E::load_raw(p.q_bias, (size_t)g * p.N + nc);
-        const unsigned char* tb = (const unsigned char*)(tab + (size_t)lt * 128);
-        acc += E::from_raw(braw) * xsum[lt];
-#pragma unroll
-        for (int b = 0; b < kLutgemmMaxBits; ++b) {
-            if ((uint32_t)b < p.bits) acc += E::from_raw(araw[b]) * lutgemm_word(tb, w[b], m);
-        }
+    const uint32_t tab_lds = (uint32_t)(uintptr_t)(DD_LDS_AS float*)tab;    // LDS byte address of the tables
+    float acc;
+    switch (p.bits) {
+        case 1: acc = lutgemm_tiles<DT, 1>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 2: acc = lutgemm_tiles<DT, 2>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 3: acc = lutgemm_tiles<DT, 3>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 4: acc = lutgemm_tiles<DT, 4>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 5: acc = lutgemm_tiles<DT, 5>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 6: acc = lutgemm_tiles<DT, 6>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        case 7: acc = lutgemm_tiles<DT, 7>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
+        default: acc = lutgemm_tiles<DT, 8>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
     }
     part[wave * 64u + lane] = acc;
     __syncthreads();
