@@ -102,7 +102,7 @@ def time_graph(torch, graph, steps, warmup):
 # HBM traffic of one launch of the roofline kernel, bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # `bench.py --leg roofline`, each scaled by what the same counter reads for the 256 MiB device copy that the
 # leg also runs (profiles/anyprec_gemv_4096x14336_pmc.md holds the runs); None = not measured for this build
-MEASURED_TRAFFIC = {"anyprec_kernel<fp16,3> 4096->14336": 23111000}
+MEASURED_TRAFFIC = {"anyprec_kernel<fp16,3> 4096->14336": 23122000}
 
 
 def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
