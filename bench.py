@@ -288,7 +288,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32, help="decoder layers per token (32 = Llama-3-8B)")
     ap.add_argument("--k-chunk", type=int, default=32)
-    ap.add_argument("--n-tb", type=int, default=8)
+    ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--leg", choices=["all", "roofline", "kernels"], default="all",

@@ -247,6 +247,48 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     }
     const uint32_t total = hd[1];
     dec_stamp(p, blockIdx.x, 6);
+    if (total <= (uint32_t)kWave) {
+        // The usual case: at most 64 candidates.  One wave holds a candidate per lane and ranks them all-pairs
+        // against the key list read back as broadcasts; nothing here needs a workgroup barrier (the other
+        // waves go straight to the barrier that precedes the fetch).
+        if (wave == 0) {
+            uint32_t mykey = 0xFFFFFFFFu;                  // padding: never smaller than a real key
+            float xs = 0.f;
+            if (lane < total) {
+                xs = cx[lane];
+                const float ca = __builtin_fabsf(xs);
+                uint32_t bkt = 0;
+#pragma unroll
+                for (int i = 0; i < kBuckets; ++i) bkt += (ca < p.floors[i]) ? 1u : 0u;
+                mykey = (bkt << 10) | key[lane];
+            }
+            key[lane] = mykey;
+            uint32_t pos = 0;
+            const u32x4* kp = (const u32x4*)key;
+            // 32 keys per step, all reads of a step in flight together (the padding keys count nothing)
+#pragma unroll 1
+            for (uint32_t h = 0; h * 32u < total; ++h) {
+                u32x4 k4[8];
+#pragma unroll
+                for (int v = 0; v < 8; ++v) k4[v] = kp[h * 8u + v];
+#pragma unroll
+                for (int v = 0; v < 8; ++v)
+                    pos += (k4[v][0] < mykey) + (k4[v][1] < mykey) + (k4[v][2] < mykey) + (k4[v][3] < mykey);
+            }
+            if (lane < total && pos < kc) {
+                const uint32_t ch = lo + (mykey & 1023u);
+                const uint32_t slot = t_local * p.k_chunk + pos;
+                lrows[slot] = (int32_t)ch;
+                lacts[slot] = xs;
+                if (write_global) {
+                    p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
+                    E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
+                }
+            }
+        }
+        dec_stamp(p, blockIdx.x, 7);
+        return;
+    }
     // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
     if (__builtin_amdgcn_readfirstlane(tid & ~63u) < total) {
         if (tid < total) {
