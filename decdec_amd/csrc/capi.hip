@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <vector>
 #include <string>
 #include <unordered_set>
 
@@ -589,9 +590,21 @@ int decdec_create_dec_config(uint64_t ctx_h, uint32_t k_chunk, int dtype, const 
             }
         }
     }
+    // The owned copy of the scales is kept in output order (scale of output n at index n), so that the two
+    // scales of an output pair arrive with one load: reordered_scales[j * N/8 + m] belongs to output 8 m + j.
     if (e == hipSuccess) e = hipMalloc(&c->scales_dev, sc_bytes);
-    if (e == hipSuccess)
-        e = hipMemcpy(c->scales_dev, scales, sc_bytes, scales_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        const size_t es = dtype_size(dtype);
+        std::vector<unsigned char> in(sc_bytes), nat(sc_bytes);
+        if (scales_on_device) e = hipMemcpy(in.data(), scales, sc_bytes, hipMemcpyDeviceToHost);
+        else memcpy(in.data(), scales, sc_bytes);
+        if (e == hipSuccess) {
+            for (uint32_t j = 0; j < 8; ++j)
+                for (uint32_t m = 0; m < c->M; ++m)
+                    memcpy(&nat[((size_t)8 * m + j) * es], &in[((size_t)j * c->M + m) * es], es);
+            e = hipMemcpy(c->scales_dev, nat.data(), sc_bytes, hipMemcpyHostToDevice);
+        }
+    }
     if (e == hipSuccess) e = hipEventCreateWithFlags(&c->e1, hipEventDisableTiming);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&c->e2, hipEventDisableTiming);
     int rc = kOk;

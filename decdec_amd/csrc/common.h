@@ -32,6 +32,12 @@ template <> struct Elem<kFP32> {
     // storage bits of element i, and their value (lets a caller request a value long before it converts it)
     static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint32_t*)p)[i]; }
     static __device__ __forceinline__ float from_raw(uint32_t r) { return __uint_as_float(r); }
+    // storage bits of the even-aligned pair (i, i + 1) and their values
+    static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
+        const u32x2 v = *(const u32x2*)((const uint32_t*)p + i); a = v[0]; b = v[1];
+    }
+    static __device__ __forceinline__ float from_raw2_lo(uint32_t a, uint32_t) { return __uint_as_float(a); }
+    static __device__ __forceinline__ float from_raw2_hi(uint32_t, uint32_t b) { return __uint_as_float(b); }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((float*)p)[i] = v; }
     // Atomically add (v0, v1) to out[i], out[i+1]; i is even.
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
@@ -75,6 +81,11 @@ template <> struct Elem<kFP16> {
     static __device__ __forceinline__ float from_raw(uint32_t r) {
         const uint16_t h = (uint16_t)r; _Float16 v; __builtin_memcpy(&v, &h, 2); return (float)v;
     }
+    static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
+        a = *(const uint32_t*)((const uint16_t*)p + i); b = 0u;
+    }
+    static __device__ __forceinline__ float from_raw2_lo(uint32_t a, uint32_t) { return from_raw(a & 0xFFFFu); }
+    static __device__ __forceinline__ float from_raw2_hi(uint32_t a, uint32_t) { return from_raw(a >> 16); }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
         half2_t v = {(_Float16)v0, (_Float16)v1};
@@ -94,6 +105,11 @@ template <> struct Elem<kBF16> {
     static __device__ __forceinline__ float load(const void* p, size_t i) { return bf16_bits_to_f32(((const uint16_t*)p)[i]); }
     static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint16_t*)p)[i]; }
     static __device__ __forceinline__ float from_raw(uint32_t r) { return bf16_bits_to_f32((uint16_t)r); }
+    static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
+        a = *(const uint32_t*)((const uint16_t*)p + i); b = 0u;
+    }
+    static __device__ __forceinline__ float from_raw2_lo(uint32_t a, uint32_t) { return __uint_as_float(a << 16); }
+    static __device__ __forceinline__ float from_raw2_hi(uint32_t a, uint32_t) { return __uint_as_float(a & 0xFFFF0000u); }
     static __device__ __forceinline__ void store(void* p, size_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
     static __device__ __forceinline__ void atomic_add2(void* out, size_t i, float v0, float v1) {
         short2_t v = {(short)f32_to_bf16_bits(v0), (short)f32_to_bf16_bits(v1)};

@@ -25,7 +25,7 @@ namespace decdec {
 
 struct DecParams {
     const uint32_t* residual;   // [K][M] u32 words, host-mapped (zero-copy) or device memory
-    const void* scales;         // reordered_scales[N], device memory, dtype of the activations
+    const void* scales;         // scale of output n at index n (the library's own copy), device memory, dtype of the activations
     const void* x;              // activations [K]
     int32_t* sel_rows;          // context scratch: selected channel indices
     void* sel_acts;             // context scratch: selected activations
@@ -384,8 +384,7 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
             const uint32_t t = tid + (uint32_t)q * kDecThreads;
             const uint32_t m = (sb0 + (t >> 8)) * kWave + (t & 63u), jp = (t >> 6) & 3u;
             const uint32_t mc = ((t < SB * 256u) && (m < p.M)) ? m : 0u;     // unconditional loads, clamped index
-            sc0[q] = E::load_raw(p.scales, (size_t)(2 * jp) * p.M + mc);
-            sc1[q] = E::load_raw(p.scales, (size_t)(2 * jp + 1) * p.M + mc);
+            E::load_raw2(p.scales, (size_t)8 * mc + 2 * jp, sc0[q], sc1[q]);
         }
 
         if (col_ok) {
@@ -395,7 +394,8 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
                 uint32_t data[U];
                 float act[U];
                 int32_t row[U];
-                // all list entries first (one LDS round trip), then the requests
+                // all list entries first (one LDS round trip), then the requests; entries are the same in
+                // every lane, so they live in scalar registers
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const uint32_t rr = r + (uint32_t)u * RL;
@@ -403,14 +403,13 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
                     const uint32_t ri = valid ? rr : 0u;
                     const int32_t rw = lrows[ri];
                     const float a = lacts[ri];
-                    row[u] = valid ? rw : -1;
-                    act[u] = (valid && rw >= 0) ? a : 0.f;
+                    row[u] = __builtin_amdgcn_readfirstlane(valid ? rw : -1);
+                    act[u] = __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(a)));
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const int32_t rw = __builtin_amdgcn_readfirstlane(row[u]);   // wave-uniform by construction
-                    if (rw >= 0) data[u] = base[(size_t)rw * p.M];
-                    else data[u] = 0x88888888u;                                  // nibble 8 == value 0
+                    if (row[u] >= 0) data[u] = base[(size_t)row[u] * p.M];
+                    else { data[u] = 0x88888888u; act[u] = 0.f; }                    // nibble 8 == value 0
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -440,7 +439,7 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
             }
             uint32_t r0 = sc0[q], r1 = sc1[q];
             asm volatile("" : "+v"(r0), "+v"(r1));        // first use of the scales: here, not earlier
-            E::atomic_add2(p.out, (size_t)8 * m + 2 * jp, v0 * E::from_raw(r0), v1 * E::from_raw(r1));
+            E::atomic_add2(p.out, (size_t)8 * m + 2 * jp, v0 * E::from_raw2_lo(r0, r1), v1 * E::from_raw2_hi(r0, r1));
         }
         dec_stamp(p, bid, 3);
         __syncthreads();                                 // red is reused by the next batch
