@@ -105,6 +105,30 @@ def pack_sqllm(idx: torch.Tensor, bits: int) -> torch.Tensor:
     return _to_int32(out.reshape(N, K // 32 * 3)).t().contiguous()
 
 
+def unpack_sqllm(qweight: torch.Tensor, bits: int) -> torch.Tensor:
+    """int32 [K*bits/32, N] -> idx int64 [N, K] (inverse of pack_sqllm)."""
+    assert bits in (3, 4)
+    w = qweight.long().t() & 0xFFFFFFFF                                       # [N, K*bits/32]
+    N = w.shape[0]
+    if bits == 4:
+        shifts = 4 * torch.arange(8, device=w.device, dtype=torch.int64)
+        return ((w[:, :, None] >> shifts) & 0xF).reshape(N, -1)
+    g = w.reshape(N, -1, 3)
+    out = torch.empty((N, g.shape[1], 32), dtype=torch.int64, device=w.device)
+    for j in range(32):
+        k, off = divmod(3 * j, 32)
+        v = g[:, :, k] >> off
+        if off + 3 > 32:
+            v = v | (g[:, :, k + 1] << (32 - off))
+        out[:, :, j] = v & 7
+    return out.reshape(N, -1)
+
+
+def dequant_sqllm(qweight: torch.Tensor, lut: torch.Tensor, bits: int) -> torch.Tensor:
+    """Dense [N, K] weight of a SqueezeLLM layer, in the LUT's dtype (reference evaluation/evaltools.py:583-645)."""
+    return dequant_lut(unpack_sqllm(qweight, bits), lut)
+
+
 # ------------------------------------------------------------------------------------------------
 # LUT-GEMM binary-coding format (reference decdec_setup/llm-awq/quantize/qmodule.py:61-92,
 # quantizer.py:216-258)

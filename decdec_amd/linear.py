@@ -24,6 +24,7 @@ class DECLinear(nn.Module):
         self.q_residual = None
         self.scales = None
         self.thresholds = None
+        self.external_zero = False      # True: the owner of `output` clears it before every decode step
 
     def load_dec_data(self, q_residual, scales, thresholds):
         assert q_residual.dtype == torch.int
@@ -79,7 +80,8 @@ class APLinear(DECLinear):
             if self.bias is not None:
                 out += self.bias
             return out
-        self.output.zero_()
+        if not self.external_zero:
+            self.output.zero_()
         if self.dec_config is None:
             ext.anyprec_gemv(x, self.output, self.qweight, self.lut, self.bitwidth)
         else:
@@ -117,7 +119,8 @@ class LUTGEMMLinear(DECLinear):
             if self.bias is not None:
                 out += self.bias
             return out
-        self.output.zero_()
+        if not self.external_zero:
+            self.output.zero_()
         if self.dec_config is None:
             ext.lutgemm_gemv(x, self.output, self.qweight, self.alpha, self.q_bias, self.bitwidth, self.group_size)
         else:
@@ -141,9 +144,19 @@ class SQLLMLinear(DECLinear):
             self.bias = None
         self.output = torch.zeros((1, 1, out_features), dtype=dtype, device=device)
 
+    def gemm(self, x):
+        weight = formats.dequant_sqllm(self.qweight, self.lut, self.bitwidth)
+        return torch.matmul(x, weight.T)
+
     def forward(self, x, **kwargs):
-        assert x.shape[0] == 1 and x.shape[1] == 1, "SQLLMLinear implements the decode path only"
-        self.output.zero_()
+        assert x.shape[0] == 1
+        if x.shape[1] > 1:
+            out = self.gemm(x)
+            if self.bias is not None:
+                out += self.bias
+            return out
+        if not self.external_zero:
+            self.output.zero_()
         if self.dec_config is None:
             ext.sqllm_gemv(x, self.output, self.qweight, self.lut, self.bitwidth)
         else:
