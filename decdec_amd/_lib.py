@@ -50,6 +50,9 @@ SIGNATURES = {
     "decdec_dummy_anyprec": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
     "decdec_dummy_lutgemm": [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
     "decdec_dummy_sqllm": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
+    "decdec_rope_cache_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp],
+    "decdec_decode_attention": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp],
+    "decdec_silu_mul": [_vp, _vp, _i32, _u32, _vp],
     "decdec_debug_read_trace": [ctypes.POINTER(_u64), _i32],
     "decdec_bucket_floors": [_f32, _f32, _i32, ctypes.POINTER(_f32)],
     "decdec_reference_geometry": [_u32, _u32, _u32, _u32, _i32, _u32, ctypes.POINTER(ConfigInfo)],

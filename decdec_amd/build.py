@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "obj")
 LIB_PATH = os.path.join(HERE, "libdecdec_hip.so")
-SOURCES = ["k_dec.hip", "k_anyprec.hip", "k_lutgemm.hip", "k_sqllm.hip", "capi.hip"]
+SOURCES = ["k_dec.hip", "k_anyprec.hip", "k_lutgemm.hip", "k_sqllm.hip", "k_decode.hip", "capi.hip"]
 ARCH = "gfx950"
 
 # -packed-fp32-ops switches the packed-FP32 VALU forms off for the device pass (the host pass

@@ -829,4 +829,41 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* mat, const v
                         [&](hipStream_t sub) { return launch_sqllm(dtype, pl.p, pl.d, sub); });
 }
 
+// ---------------------------------------------------------------- decode-step helpers
+int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos_device,
+                             void* q_out, void* k_cache, void* v_cache, int dtype, uint32_t n_head,
+                             uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(qkv && cos_table && sin_table && pos_device && q_out && k_cache && v_cache, "null pointer argument");
+    DD_CHECK(n_head >= 1 && n_kv_head >= 1 && n_head % n_kv_head == 0, "n_head must be a multiple of n_kv_head");
+    DD_CHECK(head_dim >= 2 && head_dim % 2 == 0 && max_seq >= 1, "head_dim must be even and max_seq positive");
+    RopeCacheParams p{qkv, cos_table, sin_table, (const long long*)pos_device, q_out, k_cache, v_cache,
+                      n_head, n_kv_head, head_dim, max_seq};
+    DD_HIP(launch_rope_cache(dtype, p, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                            void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                            uint32_t max_seq, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(q && k_cache && v_cache && pos_device && out, "null pointer argument");
+    DD_CHECK(n_head >= 1 && n_kv_head >= 1 && n_head % n_kv_head == 0, "n_head must be a multiple of n_kv_head");
+    DD_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128, got %u", head_dim);
+    DD_CHECK(max_seq >= 1, "max_seq must be positive");
+    DD_CHECK(((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0, "caches must be 16-byte aligned");
+    AttentionParams p{q, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
+                      1.0f / std::sqrt((float)head_dim)};
+    DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(gate_up && out, "null pointer argument");
+    if (n == 0) return kOk;
+    DD_HIP(launch_silu_mul(dtype, gate_up, out, n, (hipStream_t)stream));
+    return kOk;
+}
+
 }  // extern "C"

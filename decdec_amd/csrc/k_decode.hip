@@ -1,0 +1,163 @@
+// Decode-step helpers around the linear layers: rotary embedding + KV-cache append, grouped-query
+// attention of one new token over the cache, and the gated activation of the feed-forward block.
+// The reference leaves these to torch.compile (end-to-end/generate.py); here they are three small kernels
+// so that a captured decode step is a short chain of launches.  Token position comes from device memory:
+// a captured step advances it on the device and is replayed unchanged.
+#include "launch.h"
+
+namespace decdec {
+
+template <int DT>
+__global__ __launch_bounds__(256) void rope_cache_kernel(const RopeCacheParams p) {
+    using E = Elem<DT>;
+    const uint32_t D = p.head_dim, half = D / 2;
+    const uint32_t pairs = (p.n_head + p.n_kv) * half, vals = p.n_kv * D;
+    const uint32_t t = blockIdx.x * blockDim.x + threadIdx.x;
+    const long long pos64 = *p.pos;
+    if (pos64 < 0 || pos64 >= (long long)p.max_seq) return;            // nothing may be written outside the cache
+    const uint32_t pos = (uint32_t)pos64;
+    if (t < pairs) {
+        const uint32_t head = t / half, i = t % half;
+        const float x1 = E::load(p.qkv, (size_t)head * D + i), x2 = E::load(p.qkv, (size_t)head * D + i + half);
+        const float c = E::load(p.cos_table, (size_t)pos * D + i), s = E::load(p.sin_table, (size_t)pos * D + i);
+        const float y1 = x1 * c - x2 * s, y2 = x2 * c + x1 * s;
+        if (head < p.n_head) {
+            E::store(p.q_out, (size_t)head * D + i, y1);
+            E::store(p.q_out, (size_t)head * D + i + half, y2);
+        } else {
+            const size_t base = ((size_t)(head - p.n_head) * p.max_seq + pos) * D;
+            E::store(p.k_cache, base + i, y1);
+            E::store(p.k_cache, base + i + half, y2);
+        }
+    } else if (t < pairs + vals) {
+        const uint32_t j = t - pairs, kvh = j / D, d = j % D;
+        const float v = E::load(p.qkv, (size_t)(p.n_head + p.n_kv) * D + j);
+        E::store(p.v_cache, ((size_t)kvh * p.max_seq + pos) * D + d, v);
+    }
+}
+
+// Sum over the LPP lanes that share a cache position (LPP = 8 or 16 neighbouring lanes).
+template <int LPP>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_read<0xB1, 0xF>(v);                     // quad_perm [1,0,3,2]
+    v += dpp_read<0x4E, 0xF>(v);                     // quad_perm [2,3,0,1]
+    if constexpr (LPP == 8) {
+        v += dpp_read<0x141, 0xF>(v);                // row_half_mirror: the other quad of the half row
+    } else {
+        v += dpp_read<0x124, 0xF>(v);                // row_ror 4
+        v += dpp_read<0x128, 0xF>(v);                // row_ror 8
+    }
+    return v;
+}
+
+// One workgroup per query head.  A group of D/8 lanes owns a cache position (16 bytes of K and of V per
+// lane); a wave visits 64 / (D/8) positions per step, the 16 waves interleave, every group keeps its own
+// running maximum / sum / output (online softmax), and the groups are merged through LDS at the end.
+template <int DT, int D>
+__global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionParams p) {
+    using E = Elem<DT>;
+    constexpr int LPP = D / 8, PPW = 64 / LPP, NG = 16 * PPW;
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* pm = (float*)smem;               // [NG]
+    float* pl = pm + NG;                    // [NG]
+    float* po = pl + NG;                    // [NG][D]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t sub = lane / LPP, dl = lane % LPP;
+    const uint32_t h = blockIdx.x, kvh = h / (p.n_head / p.n_kv);
+    long long pos64 = *p.pos;
+    if (pos64 < 0) pos64 = 0;
+    const uint32_t len = (uint32_t)((pos64 + 1 < (long long)p.max_seq) ? pos64 + 1 : (long long)p.max_seq);
+    float q[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = E::load(p.q, (size_t)h * D + 8 * dl + e) * p.scale;
+    float m = -__builtin_inff(), l = 0.f, o[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = 0.f;
+    const uint16_t* kc = (const uint16_t*)p.k_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
+    const uint16_t* vc = (const uint16_t*)p.v_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
+    for (uint32_t p0 = wave * PPW; p0 < len; p0 += 16 * PPW) {
+        const uint32_t pp = p0 + sub;
+        const bool valid = pp < len;
+        const uint32_t ppc = valid ? pp : len - 1u;
+        const u32x4 kr = *(const u32x4*)(kc + (size_t)ppc * D);
+        const u32x4 vr = *(const u32x4*)(vc + (size_t)ppc * D);
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            s += q[2 * e] * E::from_raw(kr[e] & 0xFFFFu);
+            s += q[2 * e + 1] * E::from_raw(kr[e] >> 16);
+        }
+        s = group_sum<LPP>(s);
+        if (valid) {
+            const float mn = s > m ? s : m;
+            const float corr = __expf(m - mn), pr = __expf(s - mn);        // m = -inf: corr = 0
+            l = l * corr + pr;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                o[2 * e] = o[2 * e] * corr + pr * E::from_raw(vr[e] & 0xFFFFu);
+                o[2 * e + 1] = o[2 * e + 1] * corr + pr * E::from_raw(vr[e] >> 16);
+            }
+            m = mn;
+        }
+    }
+    const uint32_t g = wave * PPW + sub;
+    if (dl == 0) { pm[g] = m; pl[g] = l; }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) po[(size_t)g * D + 8 * dl + e] = o[e];
+    __syncthreads();
+    if (tid < (uint32_t)D) {
+        float M = -__builtin_inff();
+        for (int i = 0; i < NG; ++i) M = pm[i] > M ? pm[i] : M;
+        float L = 0.f, O = 0.f;
+        for (int i = 0; i < NG; ++i) {
+            const float w = (pm[i] == -__builtin_inff()) ? 0.f : __expf(pm[i] - M);
+            L += pl[i] * w;
+            O += po[(size_t)i * D + tid] * w;
+        }
+        E::store(p.out, (size_t)h * D + tid, O / L);
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ gate_up, void* __restrict__ out, uint32_t n) {
+    using E = Elem<DT>;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float a = E::load(gate_up, i), b = E::load(gate_up, (size_t)n + i);
+    E::store(out, i, a / (1.f + __expf(-a)) * b);
+}
+
+hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s) {
+    const uint32_t threads = (p.n_head + p.n_kv) * (p.head_dim / 2) + p.n_kv * p.head_dim;
+    const dim3 grid((threads + 255) / 256), block(256);
+    if (dt == kFP16) hipLaunchKernelGGL((rope_cache_kernel<kFP16>), grid, block, 0, s, p);
+    else if (dt == kBF16) hipLaunchKernelGGL((rope_cache_kernel<kBF16>), grid, block, 0, s, p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+size_t decode_attention_lds_bytes(uint32_t head_dim) {
+    const size_t ng = 16 * (64 / (head_dim / 8));
+    return ng * (head_dim + 2) * sizeof(float);
+}
+
+hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s) {
+    const dim3 grid(p.n_head), block(1024);
+    const size_t lds = decode_attention_lds_bytes(p.head_dim);
+    if (dt == kFP16 && p.head_dim == 128) hipLaunchKernelGGL((decode_attention_kernel<kFP16, 128>), grid, block, lds, s, p);
+    else if (dt == kFP16 && p.head_dim == 64) hipLaunchKernelGGL((decode_attention_kernel<kFP16, 64>), grid, block, lds, s, p);
+    else if (dt == kBF16 && p.head_dim == 128) hipLaunchKernelGGL((decode_attention_kernel<kBF16, 128>), grid, block, lds, s, p);
+    else if (dt == kBF16 && p.head_dim == 64) hipLaunchKernelGGL((decode_attention_kernel<kBF16, 64>), grid, block, lds, s, p);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, hipStream_t s) {
+    const dim3 grid((n + 255) / 256), block(256);
+    if (dt == kFP16) hipLaunchKernelGGL((silu_mul_kernel<kFP16>), grid, block, 0, s, gate_up, out, n);
+    else if (dt == kBF16) hipLaunchKernelGGL((silu_mul_kernel<kBF16>), grid, block, 0, s, gate_up, out, n);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+}  // namespace decdec

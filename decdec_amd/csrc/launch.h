@@ -32,4 +32,28 @@ hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
 hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
                             const SqllmParams& gp, const LaunchDims& d, hipStream_t s);
 
+// Decode-step helpers (k_decode.hip).  `pos` points at the token position in device memory.
+struct RopeCacheParams {
+    const void* qkv;                 // [(n_head + 2 n_kv) * head_dim]: query heads, key heads, value heads
+    const void* cos_table;           // [max_seq][head_dim]
+    const void* sin_table;
+    const long long* pos;
+    void* q_out;                     // [n_head * head_dim], rotated queries
+    void* k_cache;                   // [n_kv][max_seq][head_dim]
+    void* v_cache;
+    uint32_t n_head, n_kv, head_dim, max_seq;
+};
+struct AttentionParams {
+    const void* q;                   // [n_head * head_dim]
+    const void* k_cache;
+    const void* v_cache;
+    const long long* pos;            // attends cache positions 0 .. *pos
+    void* out;                       // [n_head * head_dim]
+    uint32_t n_head, n_kv, head_dim, max_seq;
+    float scale;
+};
+hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
+hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);
+hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, hipStream_t s);
+
 }  // namespace decdec

@@ -1,0 +1,45 @@
+"""Decode-step helpers of the library (rotary embedding + KV-cache append, one-token grouped-query
+attention, gated activation) as functions on torch tensors.  They raise if the HIP library is missing;
+there is no fallback."""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from .ext import _check, _dt, _ptr, _stream
+
+
+def _half_cuda(*ts):
+    for t in ts:
+        _check(t.is_cuda and t.is_contiguous(), "tensors must be contiguous CUDA tensors")
+        _check(t.dtype == ts[0].dtype and t.dtype in (torch.float16, torch.bfloat16), "tensors must share an fp16 / bf16 dtype")
+
+
+def rope_cache_update(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor, pos: torch.Tensor,
+                      q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, n_head: int, n_kv_head: int) -> None:
+    """qkv [(n_head + 2 n_kv_head) * D]; tables [max_seq, D]; pos int64 [1] on the device; caches [1, n_kv_head, max_seq, D]."""
+    _half_cuda(qkv, cos_table, sin_table, q_out, k_cache, v_cache)
+    _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64 on the device")
+    D, max_seq = k_cache.shape[-1], k_cache.shape[-2]
+    _check(qkv.numel() == (n_head + 2 * n_kv_head) * D and q_out.numel() == n_head * D, "qkv / q_out size mismatch")
+    _check(k_cache.numel() == n_kv_head * max_seq * D and v_cache.shape == k_cache.shape, "cache shape mismatch")
+    _check(tuple(cos_table.shape) == (max_seq, D) and tuple(sin_table.shape) == (max_seq, D), "rotary tables must be [max_seq, head_dim]")
+    _lib.check(_lib.load().decdec_rope_cache_update(_ptr(qkv), _ptr(cos_table), _ptr(sin_table), _ptr(pos), _ptr(q_out),
+                                                    _ptr(k_cache), _ptr(v_cache), _dt(qkv), n_head, n_kv_head, D, max_seq, _stream()))
+
+
+def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor,
+                     out: torch.Tensor, n_head: int, n_kv_head: int) -> None:
+    _half_cuda(q, k_cache, v_cache, out)
+    _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64 on the device")
+    D, max_seq = k_cache.shape[-1], k_cache.shape[-2]
+    _check(q.numel() == n_head * D and out.numel() == n_head * D, "q / out size mismatch")
+    _check(k_cache.numel() == n_kv_head * max_seq * D and v_cache.shape == k_cache.shape, "cache shape mismatch")
+    _lib.check(_lib.load().decdec_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(out), _dt(q),
+                                                   n_head, n_kv_head, D, max_seq, _stream()))
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    _half_cuda(gate_up, out)
+    _check(gate_up.numel() == 2 * out.numel(), "gate_up must hold twice as many elements as out")
+    _lib.check(_lib.load().decdec_silu_mul(_ptr(gate_up), _ptr(out), _dt(out), out.numel(), _stream()))

@@ -5,7 +5,9 @@ Counterpart of the reference's end-to-end/model.py (a gpt-fast style Llama / Phi
 ``load_dec_data`` / ``create_dec_context`` / ``set_dec_config`` / ``update_dec_config`` with the
 reference's meaning (k_chunks = [qkv, o, gate_up, down]).  Everything that is not a linear layer is
 plain torch: this file exists to drive the linear-layer hot path from a real decode step, not to be a
-model zoo.  A decode step touches only static buffers, so it can be captured in a HIP graph.
+model zoo.  A decode step touches only static buffers, so it can be captured in a HIP graph; on the GPU
+its rotary embedding, cache append, attention and gated activation run on the library's helper kernels
+(``decode_ops``), a prefill or CPU pass on torch ops.
 """
 from __future__ import annotations
 
@@ -116,10 +118,21 @@ class Attention(nn.Module):
         self.kv_cache: Optional[KVCache] = None
         self.n_head, self.n_local_heads, self.head_dim, self.dim = config.n_head, config.n_local_heads, config.head_dim, config.dim
 
-    def forward(self, x: torch.Tensor, mask: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, input_pos: torch.Tensor):
+    def forward(self, x: torch.Tensor, mask: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, input_pos: torch.Tensor,
+                rope_tables_full=None):
         B, S, _ = x.shape
         kv = self.n_local_heads * self.head_dim
         qkv = self.wqkv(x)
+        if rope_tables_full is not None:
+            # one-token step on the library's helper kernels: rotate + append to the cache, then attend
+            from . import decode_ops
+            q = torch.empty(self.dim, dtype=x.dtype, device=x.device)
+            decode_ops.rope_cache_update(qkv.view(-1), rope_tables_full[0], rope_tables_full[1], input_pos, q,
+                                         self.kv_cache.k_cache, self.kv_cache.v_cache, self.n_head, self.n_local_heads)
+            y = torch.empty(1, 1, self.dim, dtype=x.dtype, device=x.device)
+            decode_ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, y,
+                                        self.n_head, self.n_local_heads)
+            return self.wo(y)
         # RoPE on the query and key heads in one pass (they are neighbours in the fused projection)
         nqk = self.n_head + self.n_local_heads
         qk = apply_rope(qkv[..., :self.dim + kv].view(B, S, nqk, self.head_dim).transpose(1, 2), cos, sin)
@@ -140,8 +153,14 @@ class FeedForward(nn.Module):
         self.w1w3 = linear_class(config.dim, 2 * self.inter, bias=False, **linear_kwargs)
         self.w2 = linear_class(self.inter, config.dim, bias=False, **linear_kwargs)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
-        a, b = self.w1w3(x).split([self.inter, self.inter], dim=-1)
+    def forward(self, x: torch.Tensor, helper_kernels: bool = False) -> torch.Tensor:
+        gu = self.w1w3(x)
+        if helper_kernels:
+            from . import decode_ops
+            act = torch.empty(1, 1, self.inter, dtype=x.dtype, device=x.device)
+            decode_ops.silu_mul(gu.view(-1), act.view(-1))
+            return self.w2(act)
+        a, b = gu.split([self.inter, self.inter], dim=-1)
         return self.w2(F.silu(a) * b)
 
 
@@ -153,9 +172,9 @@ class TransformerBlock(nn.Module):
         self.input_layernorm = RMSNorm(config.dim, config.norm_eps)
         self.post_attention_layernorm = RMSNorm(config.dim, config.norm_eps)
 
-    def forward(self, x, mask, cos, sin, input_pos):
-        h = x + self.attention(self.input_layernorm(x), mask, cos, sin, input_pos)
-        return h + self.feed_forward(self.post_attention_layernorm(h))
+    def forward(self, x, mask, cos, sin, input_pos, rope_tables_full=None):
+        h = x + self.attention(self.input_layernorm(x), mask, cos, sin, input_pos, rope_tables_full)
+        return h + self.feed_forward(self.post_attention_layernorm(h), rope_tables_full is not None)
 
     def dec_linears(self):
         """The four compensated linears in the order of the k_chunk lists: qkv, o, gate_up, down."""
@@ -176,6 +195,9 @@ class Transformer(nn.Module):
         self.output = nn.Linear(config.dim, config.vocab_size, bias=False, dtype=dtype, device=device)
         self.max_batch_size = self.max_seq_length = -1
         self.dec_contexts = []
+        # one-token steps use the library's rotary / attention / activation kernels instead of torch ops
+        self.decode_kernels = (torch.device(device).type == "cuda" and dtype in (torch.float16, torch.bfloat16)
+                               and config.head_dim in (64, 128))
         self.to(device)
         for m in self.modules():
             if isinstance(m, RMSNorm):
@@ -217,9 +239,14 @@ class Transformer(nn.Module):
         assert self.max_seq_length > 0, "Caches must be initialized first"
         if idx.shape[1] == 1 and getattr(self, "output_arena", None) is not None:
             self.output_arena.zero_()
+        x = self.tok_embeddings(idx)
+        if self.decode_kernels and idx.shape == (1, 1) and x.is_cuda:
+            full = (self.rope_cos, self.rope_sin)
+            for layer in self.layers:
+                x = layer(x, None, None, None, input_pos, full)
+            return self.output(self.norm(x))
         mask = self.causal_mask.index_select(0, input_pos)                     # [S, max_seq]
         cos, sin = self.rope_cos.index_select(0, input_pos), self.rope_sin.index_select(0, input_pos)
-        x = self.tok_embeddings(idx)
         for layer in self.layers:
             x = layer(x, mask, cos, sin, input_pos)
         return self.output(self.norm(x))

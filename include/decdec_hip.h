@@ -143,6 +143,26 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
                        int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
                        int dummy_cu, int64_t dummy_iters, void* stream);
 
+/* Decode-step helpers for a caller that drives the linear layers from a captured decode step (the
+ * reference leaves these operations to torch.compile, end-to-end/generate.py; they have no counterpart in
+ * its extension).  All tensors are fp16 or bf16 in device memory; `pos_device` points at the token position
+ * (int64) in DEVICE memory, so a captured step can advance it on the device.
+ *   decdec_rope_cache_update: qkv = [query heads | key heads | value heads] of one token; rotates pair
+ *     (i, i + head_dim/2) of every query and key head by cos/sin_table[pos][i] (tables [max_seq][head_dim]),
+ *     writes the rotated queries to q_out and the rotated keys and the values into row `pos` of the caches
+ *     ([n_kv_head][max_seq][head_dim]).  A position outside [0, max_seq) writes nothing.
+ *   decdec_decode_attention: out[h] = softmax(q[h] . K[kv(h)][0..pos] / sqrt(head_dim)) V[kv(h)][0..pos],
+ *     head_dim 64 or 128, grouped-query heads (kv(h) = h / (n_head / n_kv_head)).
+ *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n. */
+int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void* sin_table,
+                             const int64_t* pos_device, void* q_out, void* k_cache, void* v_cache,
+                             int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                             uint32_t max_seq, void* stream);
+int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                            const int64_t* pos_device, void* out, int dtype, uint32_t n_head,
+                            uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream);
+int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
+
 /* Diagnostics: with option "dec_trace" = 1 every DEC workgroup stores shader-clock stamps of its
  * phases (0 start, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a
  * library-owned device buffer; this copies the first `workgroups` x 8 stamps to the host (it

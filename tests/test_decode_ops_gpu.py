@@ -1,0 +1,106 @@
+"""Decode-step helper kernels against plain fp32 torch references (these are floating-point kernels; the
+tolerance is the rounding of their 16-bit outputs)."""
+import math
+
+import pytest
+import torch
+
+from decdec_amd import decode_ops as D, generate as G
+from decdec_amd.model import apply_rope, rope_tables
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, rtol):
+    got, want = got.float(), want.float()
+    return float((got - want).abs().max()) <= rtol * float(want.abs().max()) + 1e-6
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,hd", [(8, 2, 64), (32, 8, 128), (4, 4, 128)])
+def test_rope_cache_update(H, Hkv, hd, dt):
+    S = 96
+    g = torch.Generator(device="cuda").manual_seed(0)
+    cos, sin = rope_tables(hd, S, 10000.0, "cuda")
+    cos16, sin16 = cos.to(dt), sin.to(dt)
+    kc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    vc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    for pos in (0, 5, S - 1):
+        qkv = torch.randn((H + 2 * Hkv) * hd, generator=g, device="cuda").to(dt)
+        k0, v0 = kc.clone(), vc.clone()
+        q_out = torch.empty(H * hd, dtype=dt, device="cuda")
+        p = torch.tensor([pos], device="cuda")
+        D.rope_cache_update(qkv, cos16, sin16, p, q_out, kc, vc, H, Hkv)
+        heads = qkv.float().view(H + 2 * Hkv, hd)
+        want = apply_rope(heads[:H + Hkv].view(1, H + Hkv, 1, hd), cos16[pos:pos + 1].float(), sin16[pos:pos + 1].float())[0, :, 0]
+        rt = 2e-2 if dt == torch.bfloat16 else 3e-3
+        assert _close(q_out.view(H, hd), want[:H], rt)
+        assert _close(kc[0, :, pos], want[H:], rt)
+        assert torch.equal(vc[0, :, pos], heads[H + Hkv:].to(dt))
+        keep = torch.ones(S, dtype=torch.bool, device="cuda"); keep[pos] = False
+        assert torch.equal(kc[0][:, keep], k0[0][:, keep]) and torch.equal(vc[0][:, keep], v0[0][:, keep])
+    k0, v0 = kc.clone(), vc.clone()
+    for bad in (-1, S, S + 7):
+        D.rope_cache_update(qkv, cos16, sin16, torch.tensor([bad], device="cuda"), q_out, kc, vc, H, Hkv)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, k0) and torch.equal(vc, v0)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,hd,S", [(8, 2, 64, 256), (32, 8, 128, 2048), (4, 4, 128, 80), (40, 10, 128, 520)])
+def test_decode_attention(H, Hkv, hd, S, dt):
+    g = torch.Generator(device="cuda").manual_seed(1)
+    kc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    vc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    for pos in sorted({0, 1, 15, 16, 63, 64, S // 2 + 3, S - 1}):
+        q = (torch.randn(H * hd, generator=g, device="cuda") * 1.5).to(dt)
+        out = torch.empty(H * hd, dtype=dt, device="cuda")
+        D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out, H, Hkv)
+        k = kc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)       # [H, L, hd]
+        v = vc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)
+        att = torch.softmax(torch.einsum("hd,hld->hl", q.float().view(H, hd), k) / math.sqrt(hd), dim=-1)
+        want = torch.einsum("hl,hld->hd", att, v)
+        assert _close(out.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos,)
+    # a position beyond the cache attends the whole cache and reads nothing outside it
+    D.decode_attention(q, kc, vc, torch.tensor([S + 100], device="cuda"), out, H, Hkv)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("n", [1, 255, 14336])
+def test_silu_mul(n):
+    gu = torch.randn(2 * n, device="cuda").half() * 3
+    out = torch.empty(n, dtype=torch.float16, device="cuda")
+    D.silu_mul(gu, out)
+    want = torch.nn.functional.silu(gu[:n].float()) * gu[n:].float()
+    assert _close(out, want, 2e-3)
+
+
+def test_argument_checks():
+    a = torch.zeros(8, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="twice as many"):
+        D.silu_mul(a, a)
+    with pytest.raises(RuntimeError, match="fp16 / bf16"):
+        D.silu_mul(torch.zeros(16, device="cuda"), torch.zeros(8, device="cuda"))
+    kc = torch.zeros(1, 2, 16, 32, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="head_dim must be 64 or 128"):
+        D.decode_attention(torch.zeros(4 * 32, dtype=torch.float16, device="cuda"), kc, kc.clone(),
+                           torch.tensor([0], device="cuda"), torch.zeros(4 * 32, dtype=torch.float16, device="cuda"), 4, 2)
+
+
+def test_decode_step_on_helper_kernels_equals_the_torch_path():
+    model = G.build_model("tiny-llama-test", "sqllm", 4, seed=9)
+    model.setup_caches(1, 64)
+    assert model.decode_kernels
+    prompt = torch.randint(0, model.config.vocab_size, (1, 30), device="cuda")
+    outs = {}
+    for use in (True, False):
+        model.decode_kernels = use
+        for b in model.layers:
+            b.attention.kv_cache.k_cache.zero_(); b.attention.kv_cache.v_cache.zero_()
+        with torch.no_grad():
+            model(prompt, torch.arange(30, device="cuda"))
+            ys = [model(torch.tensor([[t]], device="cuda"), torch.tensor([30 + i], device="cuda")).float().clone()
+                  for i, t in enumerate((3, 99, 250))]
+        outs[use] = torch.stack(ys)
+    assert _close(outs[True], outs[False], 1e-2)
