@@ -54,6 +54,7 @@ struct Options {
     int sqllm_ktiles = 0;
     int dec_trace = 0;
     int anyprec_rg = 0;
+    int fused_two_per_cu = -1;  // fused launches: 1 / 0 = always / never two workgroups per compute unit, -1 = by estimate
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
@@ -71,6 +72,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "dec_trace")) return &g_opt.dec_trace;
     if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
     if (!strcmp(name, "anyprec_tile")) return &g_opt.anyprec_tile;
+    if (!strcmp(name, "fused_two_per_cu")) return &g_opt.fused_two_per_cu;
     return nullptr;
 }
 
@@ -729,6 +731,18 @@ int decdec_sqllm_gemv(const void* input, void* output, const void* mat, const vo
 }
 
 // ---------------------------------------------------------------- DEC + base GEMV
+// Which instance of a fused kernel to launch: the one that lets two workgroups share a compute unit when the
+// GEMV role is expected to outlast the DEC role by a margin.  Estimates in microseconds: DEC = its latency
+// floor (launch, activation load, selection, one host-link round trip, merge: about 8) plus the residual
+// bytes at the zero-copy rate of the link (56 GB/s); GEMV = 2 plus its weight bytes at 2.5 TB/s.
+bool fused_two_per_cu(const Config* c, double gemv_bytes) {
+    if (g_opt.fused_two_per_cu >= 0) return g_opt.fused_two_per_cu != 0;
+    const double k = (double)((uint64_t)c->k_chunk * c->K / 1024u);        // selected rows per call
+    const double dec_us = 8.0 + k * (double)c->N * 0.5 / 56e3;
+    const double gemv_us = 2.0 + gemv_bytes / 2.5e6;
+    return gemv_us > 1.25 * dec_us;
+}
+
 int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
                        int bits, int dtype, uint32_t K, uint32_t N, void* stream) {
     Config* c = get_config(h);
@@ -739,12 +753,14 @@ int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* 
     const bool have_dec = fill_dec_params(c, input, output, true, &dp) == 0;
     const bool fuse = g_opt.fusion && have_dec;
     AnyprecPlan pl;
+    const bool two = fuse && bits == 3 && fused_two_per_cu(c, (double)bits * N * K / 8.0);
     rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, fuse, &pl);
     if (rc != kOk) return rc;
     hipStream_t s = (hipStream_t)stream;
     if (fuse) {
         LaunchDims d = pl.d;
         d.lds = std::max(d.lds, c->plan.lds);
+        d.two_per_cu = two;
         DD_HIP(launch_dec_anyprec(dtype, bits, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
         return kOk;
     }
@@ -791,6 +807,7 @@ int decdec_dec_sqllm(uint64_t h, const void* input, void* output, const void* ma
     if (fuse) {
         LaunchDims d = pl.d;
         d.lds = std::max(d.lds, c->plan.lds);
+        d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
         DD_HIP(launch_dec_sqllm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
         return kOk;
     }

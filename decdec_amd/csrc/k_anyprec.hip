@@ -10,8 +10,8 @@ __global__ __launch_bounds__(1024) void anyprec_kernel(const AnyprecParams p) {
     anyprec_role<DT, BITS>(p, blockIdx.x, smem);
 }
 
-template <int DT, int BITS>
-__global__ __launch_bounds__(1024) void dec_anyprec_kernel(const DecParams dp, const uint32_t dec_blocks,
+template <int DT, int BITS, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_anyprec_kernel(const DecParams dp, const uint32_t dec_blocks,
                                                            const AnyprecParams gp) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
@@ -78,10 +78,16 @@ hipError_t launch_anyprec(int dt, int bits, const AnyprecParams& p, const Launch
 hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t dec_blocks,
                               const AnyprecParams& gp, const LaunchDims& d, hipStream_t s) {
     const dim3 grid(dec_blocks + d.grid), block(d.block);
+    if (d.two_per_cu && bits == 3) {       // only the 3-bit instances fit the register budget without spilling
+        if (dt == kFP16) hipLaunchKernelGGL((dec_anyprec_kernel<kFP16, 3, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+        else if (dt == kBF16) hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, 3, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+        else return hipErrorInvalidValue;
+        return hipGetLastError();
+    }
     if (dt == kFP16) {
-        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kFP16, B>), grid, block, d.lds, s, dp, dec_blocks, gp));
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kFP16, B, false>), grid, block, d.lds, s, dp, dec_blocks, gp));
     } else if (dt == kBF16) {
-        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, B>), grid, block, d.lds, s, dp, dec_blocks, gp));
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, B, false>), grid, block, d.lds, s, dp, dec_blocks, gp));
     } else {
         return hipErrorInvalidValue;
     }

@@ -9,8 +9,8 @@ __global__ __launch_bounds__(1024) void sqllm_kernel(const SqllmParams p) {
     sqllm_role<DT>(p, blockIdx.x, smem);
 }
 
-template <int DT>
-__global__ __launch_bounds__(1024) void dec_sqllm_kernel(const DecParams dp, const uint32_t dec_blocks,
+template <int DT, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_sqllm_kernel(const DecParams dp, const uint32_t dec_blocks,
                                                            const SqllmParams gp) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
@@ -27,7 +27,9 @@ static hipError_t sqllm_prepare() {
         hipError_t e = hipSuccess;
         auto acc = [&e](hipError_t r) { if (e == hipSuccess) e = r; };
         acc(allow_large_lds(sqllm_kernel<kFP32>)); acc(allow_large_lds(sqllm_kernel<kFP16>)); acc(allow_large_lds(sqllm_kernel<kBF16>));
-        acc(allow_large_lds(dec_sqllm_kernel<kFP32>)); acc(allow_large_lds(dec_sqllm_kernel<kFP16>)); acc(allow_large_lds(dec_sqllm_kernel<kBF16>));
+        acc(allow_large_lds(dec_sqllm_kernel<kFP32, false>));
+        acc(allow_large_lds(dec_sqllm_kernel<kFP16, false>)); acc(allow_large_lds(dec_sqllm_kernel<kFP16, true>));
+        acc(allow_large_lds(dec_sqllm_kernel<kBF16, false>)); acc(allow_large_lds(dec_sqllm_kernel<kBF16, true>));
         return e;
     }();
     return done;
@@ -48,10 +50,17 @@ hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
                               const SqllmParams& gp, const LaunchDims& d, hipStream_t s) {
     if (hipError_t e = sqllm_prepare(); e != hipSuccess) return e;
     const dim3 grid(dec_blocks + d.grid), block(d.block);
+    const bool two = d.two_per_cu && dt != kFP32;      // the fp32 instance would spill registers under the budget
     switch (dt) {
-        case kFP32: hipLaunchKernelGGL(dec_sqllm_kernel<kFP32>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
-        case kFP16: hipLaunchKernelGGL(dec_sqllm_kernel<kFP16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
-        case kBF16: hipLaunchKernelGGL(dec_sqllm_kernel<kBF16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kFP32: hipLaunchKernelGGL((dec_sqllm_kernel<kFP32, false>), grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kFP16:
+            if (two) hipLaunchKernelGGL((dec_sqllm_kernel<kFP16, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            else hipLaunchKernelGGL((dec_sqllm_kernel<kFP16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            break;
+        case kBF16:
+            if (two) hipLaunchKernelGGL((dec_sqllm_kernel<kBF16, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            else hipLaunchKernelGGL((dec_sqllm_kernel<kBF16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -12,7 +12,15 @@ struct LaunchDims {
     uint32_t grid;
     uint32_t block;
     size_t lds;
+    bool two_per_cu = false;   // fused launches: use the kernel instance held to 64 vector / 96 scalar registers
 };
+
+// A fused kernel runs 1024-thread workgroups.  Two of them share a compute unit (eight waves per SIMD) only
+// if a wave needs at most 64 vector and 96 scalar registers; the attribute makes the compiler keep to that.
+// Sharing pays when the GEMV role outlasts the DEC role (its waves then fill the whole chip); a DEC
+// workgroup that shares its unit with GEMV waves takes about a microsecond longer, so launches in which
+// DEC is the longer role use the unconstrained instance, one workgroup per unit.
+#define DD_TWO_PER_CU(on) __attribute__((amdgpu_waves_per_eu((on) ? 8 : 4, 8)))
 
 // Standalone kernels.
 hipError_t launch_dec(int dt, const DecParams& p, const LaunchDims& d, hipStream_t s);

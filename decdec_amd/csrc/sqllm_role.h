@@ -71,11 +71,13 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
         // build: this thread's column, high field = wave, low field 0..15
         {
             const u32x4 a = *(const u32x4*)lrow, b = *(const u32x4*)(lrow + 8);
-            const uint32_t d[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
             const uint32_t vh = (uint32_t)lrow[wave] << 16;
             uint32_t* dst = pair_s + (size_t)(wave * 16u) * 64 + lane;
 #pragma unroll
-            for (int lo = 0; lo < 16; ++lo) dst[lo * 64] = ((lo & 1) ? (d[lo >> 1] >> 16) : (d[lo >> 1] & 0xFFFFu)) | vh;
+            for (int lo = 0; lo < 16; ++lo) {
+                const uint32_t dw = (lo < 8) ? a[(lo >> 1) & 3] : b[(lo >> 1) & 3];     // indices are constants after unrolling
+                dst[lo * 64] = ((lo & 1) ? (dw >> 16) : (dw & 0xFFFFu)) | vh;
+            }
         }
         __syncthreads();
         uint32_t m = 0xFF00u;
@@ -102,13 +104,12 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
         // 3-bit: 64 entries; high field = wave / 2, low fields 4 (wave & 1) .. + 3
         {
             const u32x4 a = *(const u32x4*)lrow;
-            const uint32_t d[4] = {a[0], a[1], a[2], a[3]};
             const uint32_t hi = wave >> 1, lo0 = (wave & 1u) * 4u;
             const uint32_t vh = (uint32_t)lrow[hi] << 16;
             uint32_t* dst = pair_s + (size_t)(hi * 8u + lo0) * 64 + lane;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const uint32_t dw = (wave & 1u) ? d[2 + (q >> 1)] : d[q >> 1];
+                const uint32_t dw = (wave & 1u) ? a[2 + (q >> 1)] : a[q >> 1];
                 dst[q * 64] = ((q & 1) ? (dw >> 16) : (dw & 0xFFFFu)) | vh;
             }
         }

@@ -245,6 +245,37 @@ def test_dec_plus_gemv(kind, fusion, c_oracle):
     ext.destroy_dec_config(cfg)
 
 
+@pytest.mark.parametrize("kind", ["anyprec", "sqllm"])
+@pytest.mark.parametrize("K,N,k_chunk", [(4096, 4096, 4), (14336, 1032, 2), (1536, 2056, 8)])
+def test_fused_launch_with_two_workgroups_per_cu(kind, K, N, k_chunk, c_oracle):
+    """The register-budgeted instances of the fused kernels (any-precision: every wave walks over its own
+    units) against the oracle, forced on whatever the estimate would choose."""
+    from decdec_amd import _lib
+    L = make_dec_layer(K, N, seed=K + N)
+    ctx, rows, acts = _ctx(16, K, torch.float16)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+    x = L["x"].cuda()
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    _lib.set_option("fused_two_per_cu", 1)
+    try:
+        if kind == "anyprec":
+            ext.dec_anyprec(cfg, x, out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+            base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+        else:
+            idx, lut = F.quantize_uniform_rows(L["W"], 4)
+            mat = F.pack_sqllm(idx, 4)
+            ext.dec_sqllm(cfg, x, out, mat.cuda(), lut.cuda(), 4)
+            base = c_oracle.sqllm_gemv(np_of(L["x"]), mat.numpy(), np_of(lut), 4)
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_option("fused_two_per_cu", -1)
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+    want = base + c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= TOL, (mre, mae)
+    ext.destroy_dec_config(cfg)
+
+
 def test_unfused_dec_uses_caller_indices(c_oracle):
     """evaluation/evaltools.py:327-343: exact top-k indices are written into the context's row
     buffer and unfused_dec fetches those rows."""
