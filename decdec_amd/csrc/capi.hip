@@ -785,6 +785,7 @@ int decdec_dec_lutgemm(uint64_t h, const void* input, void* output, const void* 
     if (fuse) {
         LaunchDims d = pl.d;
         d.lds = std::max(d.lds, c->plan.lds);
+        d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
         DD_HIP(launch_dec_lutgemm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
         return kOk;
     }

@@ -9,9 +9,9 @@ __global__ __launch_bounds__(1024) void lutgemm_kernel(const LutgemmParams p) {
     lutgemm_role<DT>(p, blockIdx.x, smem);
 }
 
-template <int DT>
-__global__ __launch_bounds__(1024) void dec_lutgemm_kernel(const DecParams dp, const uint32_t dec_blocks,
-                                                           const LutgemmParams gp) {
+template <int DT, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_lutgemm_kernel(const DecParams dp, const uint32_t dec_blocks,
+                                                                             const LutgemmParams gp) {
     extern __shared__ __align__(16) unsigned char smem[];
     if (blockIdx.x < dec_blocks) dec_role<DT>(dp, blockIdx.x, smem);
     else lutgemm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
@@ -30,10 +30,20 @@ hipError_t launch_lutgemm(int dt, const LutgemmParams& p, const LaunchDims& d, h
 hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
                               const LutgemmParams& gp, const LaunchDims& d, hipStream_t s) {
     const dim3 grid(dec_blocks + d.grid), block(d.block);
+    const bool two = d.two_per_cu;
     switch (dt) {
-        case kFP32: hipLaunchKernelGGL(dec_lutgemm_kernel<kFP32>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
-        case kFP16: hipLaunchKernelGGL(dec_lutgemm_kernel<kFP16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
-        case kBF16: hipLaunchKernelGGL(dec_lutgemm_kernel<kBF16>, grid, block, d.lds, s, dp, dec_blocks, gp); break;
+        case kFP32:
+            if (two) hipLaunchKernelGGL((dec_lutgemm_kernel<kFP32, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            else hipLaunchKernelGGL((dec_lutgemm_kernel<kFP32, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            break;
+        case kFP16:
+            if (two) hipLaunchKernelGGL((dec_lutgemm_kernel<kFP16, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            else hipLaunchKernelGGL((dec_lutgemm_kernel<kFP16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            break;
+        case kBF16:
+            if (two) hipLaunchKernelGGL((dec_lutgemm_kernel<kBF16, true>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            else hipLaunchKernelGGL((dec_lutgemm_kernel<kBF16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
+            break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

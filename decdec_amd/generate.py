@@ -191,7 +191,7 @@ def main(argv=None):
     ap.add_argument("--algo", choices=sorted(LINEAR_CLASSES), default="sqllm")
     ap.add_argument("--bitwidth", type=int, default=4)
     ap.add_argument("--group-size", type=int, default=128)
-    ap.add_argument("--k-chunk", type=int, nargs="+", default=[8], help="one value, or four: qkv o gate_up down")
+    ap.add_argument("--k-chunk", type=int, nargs="+", default=[8], help="one value, or groups of four (qkv o gate_up down); every group is one DEC run")
     ap.add_argument("--n-tb", type=int, default=16)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--max-new-tokens", type=int, default=256)
@@ -199,7 +199,11 @@ def main(argv=None):
     ap.add_argument("--n-layer", type=int, default=None, help="fewer layers than the named model (smoke runs)")
     ap.add_argument("--no-graph", action="store_true")
     args = ap.parse_args(argv)
-    ks = args.k_chunk * 4 if len(args.k_chunk) == 1 else args.k_chunk
+    if len(args.k_chunk) == 1:
+        k_sets = [args.k_chunk * 4]
+    else:
+        assert len(args.k_chunk) % 4 == 0, "--k-chunk takes one value or groups of four (qkv o gate_up down)"
+        k_sets = [args.k_chunk[i:i + 4] for i in range(0, len(args.k_chunk), 4)]
     log = lambda s: print(s, file=sys.stderr, flush=True)
 
     model = build_model(args.model, args.algo, args.bitwidth, args.group_size, n_layer=args.n_layer)
@@ -211,17 +215,23 @@ def main(argv=None):
     log(f"base: {n / t_base:.1f} tokens/s; calibrating thresholds")
     th = calibrate_thresholds(model)
     model.load_dec_data(random_dec_data(model, th))
-    model.create_dec_context(args.n_tb, buffer_size=max(1024, max(ks) * (model.config.intermediate_size // 1024 + 1)))
-    model.set_dec_config(ks)
-    log("DEC run")
-    seq1, t_dec = generate(model, prompt, args.max_new_tokens, not args.no_graph, args.max_seq_length)
-    print(json.dumps({
-        "metric": "tokens/s, batch-1 greedy decode", "model": args.model, "n_layer": model.config.n_layer,
-        "algo": args.algo, "bitwidth": args.bitwidth, "k_chunk": ks, "n_tb": args.n_tb,
-        "prompt_len": args.prompt_len, "new_tokens": args.max_new_tokens, "graph": not args.no_graph,
-        "tokens_per_s_base": round(n / t_base, 2), "tokens_per_s_dec": round(n / t_dec, 2),
-        "ms_per_token_base": round(t_base / n * 1e3, 4), "ms_per_token_dec": round(t_dec / n * 1e3, 4),
-        "dec_slowdown_pct": round((t_dec / t_base - 1) * 100, 2), "data": "synthetic (random weights and prompt)"}))
+    k_max = max(max(ks) for ks in k_sets)
+    model.create_dec_context(args.n_tb, buffer_size=max(1024, k_max * (model.config.intermediate_size // 1024 + 1)))
+    for i, ks in enumerate(k_sets):
+        if i == 0:
+            model.set_dec_config(ks)              # pins the residuals
+        else:
+            model.update_dec_config(ks)           # same pinned residuals, new k_chunk
+        log(f"DEC run, k_chunk {ks}")
+        seq1, t_dec = generate(model, prompt, args.max_new_tokens, not args.no_graph, args.max_seq_length)
+        print(json.dumps({
+            "metric": "tokens/s, batch-1 greedy decode", "model": args.model, "n_layer": model.config.n_layer,
+            "algo": args.algo, "bitwidth": args.bitwidth, "k_chunk": ks, "n_tb": args.n_tb,
+            "prompt_len": args.prompt_len, "new_tokens": args.max_new_tokens, "graph": not args.no_graph,
+            "tokens_per_s_base": round(n / t_base, 2), "tokens_per_s_dec": round(n / t_dec, 2),
+            "ms_per_token_base": round(t_base / n * 1e3, 4), "ms_per_token_dec": round(t_dec / n * 1e3, 4),
+            "dec_slowdown_pct": round((t_dec / t_base - 1) * 100, 2), "data": "synthetic (random weights and prompt)"}),
+            flush=True)
 
 
 if __name__ == "__main__":
