@@ -54,9 +54,15 @@ struct Options {
     int sqllm_ktiles = 0;
     int dec_trace = 0;
     int anyprec_rg = 0;
+    int dec_block_waves = 16;   // waves of a standalone DEC workgroup (4 .. 16)
     int fused_two_per_cu = -1;  // fused launches: 1 / 0 = always / never two workgroups per compute unit, -1 = by estimate
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
+
+uint32_t dec_block_threads() {
+    const int w = std::min(std::max(g_opt.dec_block_waves, (int)kMinDecWaves), (int)kDecWaves);
+    return (uint32_t)w * kWave;
+}
 
 // Diagnostics: per-workgroup cycle stamps of the DEC phases (option "dec_trace").
 constexpr int kTraceBlocks = 4096;
@@ -73,6 +79,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
     if (!strcmp(name, "anyprec_tile")) return &g_opt.anyprec_tile;
     if (!strcmp(name, "fused_two_per_cu")) return &g_opt.fused_two_per_cu;
+    if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     return nullptr;
 }
 
@@ -451,7 +458,7 @@ static int two_stream(Config* c, const DecParams* dp, bool have_dec, int dtype, 
     hipStream_t sub = c->ctx->sub_stream;
     DD_HIP(hipEventRecord(c->e1, main_stream));
     if (have_dec) {
-        LaunchDims d{c->plan.cg * c->plan.sg, (uint32_t)kDecThreads, c->plan.lds};
+        LaunchDims d{c->plan.cg * c->plan.sg, dec_block_threads(), c->plan.lds};
         DD_HIP(launch_dec(dtype, *dp, d, main_stream));
     }
     DD_HIP(hipStreamWaitEvent(sub, c->e1, 0));
@@ -678,7 +685,7 @@ static int dec_common(uint64_t h, const void* input, void* output, int dtype, ui
     if (rc != kOk) return rc;
     DecParams p;
     if (fill_dec_params(c, input, output, fused_select, &p)) return kOk;
-    LaunchDims d{c->plan.cg * c->plan.sg, (uint32_t)kDecThreads, c->plan.lds};
+    LaunchDims d{c->plan.cg * c->plan.sg, dec_block_threads(), c->plan.lds};
     DD_HIP(launch_dec(dtype, p, d, (hipStream_t)stream));
     return kOk;
 }

@@ -46,14 +46,17 @@ __device__ __forceinline__ void dec_stamp(const DecParams& p, uint32_t bid, int 
     if (p.trace != nullptr && threadIdx.x == 0) p.trace[(size_t)bid * 8 + k] = __builtin_readcyclecounter();
 }
 
-constexpr int kDecThreads = 1024;
+constexpr int kDecThreads = 1024;                            // largest DEC workgroup
 constexpr int kDecWaves = kDecThreads / kWave;
+constexpr int kMinDecWaves = 4;                              // smallest: the four scanning waves
 constexpr int kMaxCand = 256;                                // fast-path candidate list capacity
 constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per thread and segment batch
 
-__host__ __device__ inline size_t dec_lds_bytes(uint32_t slots) {
-    // row list (index + activation) + selection counters/prefix + cross-wave reduction buffer
-    return (size_t)slots * 8 + 2 * 512 * 4 + (size_t)kDecWaves * 8 * kWave * 4;
+__host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves = kDecWaves) {
+    // row list (index + activation) + selection counters/prefix + the buffer shared by the cross-wave
+    // reduction ([nwaves][8][64] floats) and the partial ranks of the selection ([16][kMaxCand])
+    const size_t red = (size_t)nwaves * 8 * kWave * 4, ranks = (size_t)16 * kMaxCand * 4;
+    return (size_t)slots * 8 + 2 * 512 * 4 + (red > ranks ? red : ranks);
 }
 
 // ---- selection of one chunk ------------------------------------------------------------------
@@ -65,26 +68,39 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
                                                 int32_t* lrows, float* lacts, uint32_t* cnt, uint32_t* pre,
                                                 bool write_global) {
     using E = Elem<DT>;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6;
     const uint32_t lo = c * kChunk;
     const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
-    const bool in = tid < len;
-    const float xv = in ? E::load(p.x, lo + tid) : 0.f;
-    const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");   // NaN is a member of no bucket
+    // The chunk is 16 groups of 64 channels; wave w plays groups w, w + nw, ... (one group per wave in a
+    // 1024-thread workgroup, four in a 256-thread one).
+    constexpr int kPasses = kChunk / kWave / kMinDecWaves;
     const float myfloor = p.floors[lane & 31u];                      // lane i holds floor[i]
-    uint32_t member = 0;
-    float ce = __builtin_inff();
+    float xv[kPasses];
+    uint32_t member[kPasses];
+#pragma unroll
+    for (int ps = 0; ps < kPasses; ++ps) {
+        const uint32_t vw = (uint32_t)ps * nw + wave;                // group of this pass
+        member[ps] = 0;
+        xv[ps] = 0.f;
+        if (vw < (uint32_t)(kChunk / kWave)) {                       // uniform per wave
+            const uint32_t ch = vw * kWave + lane;
+            const bool in = ch < len;
+            xv[ps] = in ? E::load(p.x, lo + ch) : 0.f;
+            const float a = in ? __builtin_fabsf(xv[ps]) : __builtin_nanf("");   // NaN is a member of no bucket
+            float ce = __builtin_inff();
 #pragma unroll 1
-    for (int i = 0; i < kBuckets; ++i) {
-        const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
-        const bool bit = (a >= fl) && (a < ce);
-        ce = fl;
-        member |= (uint32_t)bit << i;
-        const unsigned long long m = __ballot(bit);
-        if (lane == 0) cnt[i * kDecWaves + wave] = (uint32_t)__popcll(m);
+            for (int i = 0; i < kBuckets; ++i) {
+                const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+                const bool bit = (a >= fl) && (a < ce);
+                ce = fl;
+                member[ps] |= (uint32_t)bit << i;
+                const unsigned long long m = __ballot(bit);
+                if (lane == 0) cnt[i * 16 + vw] = (uint32_t)__popcll(m);
+            }
+        }
     }
     __syncthreads();
-    if (wave == 0) {   // exclusive prefix over the 512 (bucket-major, wave-minor) counts
+    if (wave == 0) {   // exclusive prefix over the 512 (bucket-major, group-minor) counts
         uint32_t v[8], sum = 0;
 #pragma unroll
         for (int q = 0; q < 8; ++q) { v[q] = cnt[lane * 8 + q]; sum += v[q]; }
@@ -99,20 +115,26 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
         for (int q = 0; q < 8; ++q) { pre[lane * 8 + q] = run; run += v[q]; }
     }
     __syncthreads();
+#pragma unroll
+    for (int ps = 0; ps < kPasses; ++ps) {
+        const uint32_t vw = (uint32_t)ps * nw + wave;
+        if (vw >= (uint32_t)(kChunk / kWave)) continue;              // uniform per wave
+        const uint32_t ch = vw * kWave + lane;
 #pragma unroll 1
-    for (int i = 0; i < kBuckets; ++i) {
-        if (pre[i * kDecWaves] >= kc) break;                // uniform: later buckets start even later
-        const bool bit = (member >> i) & 1u;
-        const unsigned long long m = __ballot(bit);
-        if (bit) {
-            const uint32_t pos = pre[i * kDecWaves + wave] + ballot_rank(m);
-            if (pos < kc) {
-                const uint32_t slot = t_local * p.k_chunk + pos;
-                lrows[slot] = (int32_t)(lo + tid);
-                lacts[slot] = xv;
-                if (write_global) {
-                    p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)(lo + tid);
-                    E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xv);
+        for (int i = 0; i < kBuckets; ++i) {
+            if (pre[i * 16] >= kc) break;                            // uniform: later buckets start even later
+            const bool bit = (member[ps] >> i) & 1u;
+            const unsigned long long m = __ballot(bit);
+            if (bit) {
+                const uint32_t pos = pre[i * 16 + vw] + ballot_rank(m);
+                if (pos < kc) {
+                    const uint32_t slot = t_local * p.k_chunk + pos;
+                    lrows[slot] = (int32_t)(lo + ch);
+                    lacts[slot] = xv[ps];
+                    if (write_global) {
+                        p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)(lo + ch);
+                        E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xv[ps]);
+                    }
                 }
             }
         }
@@ -305,7 +327,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per wave and round
         const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
 #pragma unroll 1
-        for (uint32_t tile = wave; tile < ntiles; tile += kDecWaves) {
+        for (uint32_t tile = wave; tile < ntiles; tile += (blockDim.x >> 6)) {
             const uint32_t jg = tile % njg, iq = tile / njg;
             const uint32_t j = jg * 64u + lane;
             const uint32_t mykey = j < total ? key[j] : 0u;
@@ -359,14 +381,14 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
                                           const int32_t* lrows, const float* lacts, float* red) {
     using E = Elem<DT>;
     constexpr int U = 8;                                // residual rows in flight per wave
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6, nt = blockDim.x;
     const uint32_t seg_lo = sgid * p.segs_per_block;
     const uint32_t seg_hi = (seg_lo + p.segs_per_block) < p.nseg ? (seg_lo + p.segs_per_block) : p.nseg;
 
 #pragma unroll 1
-    for (uint32_t sb0 = seg_lo; sb0 < seg_hi; sb0 += kDecWaves) {
-        const uint32_t SB = (seg_hi - sb0) < (uint32_t)kDecWaves ? (seg_hi - sb0) : (uint32_t)kDecWaves;
-        const uint32_t RL = kDecWaves / SB;             // waves sharing one segment
+    for (uint32_t sb0 = seg_lo; sb0 < seg_hi; sb0 += nw) {
+        const uint32_t SB = (seg_hi - sb0) < nw ? (seg_hi - sb0) : nw;
+        const uint32_t RL = nw / SB;                    // waves sharing one segment
         const uint32_t ls = wave % SB, rl = wave / SB;
         const uint32_t w0 = (sb0 + ls) * kWave + lane;  // u32 column of the residual row
         const bool col_ok = (rl < RL) && (w0 < p.M);
@@ -381,7 +403,7 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
         uint32_t sc0[kMergeTasks], sc1[kMergeTasks];
 #pragma unroll
         for (int q = 0; q < kMergeTasks; ++q) {
-            const uint32_t t = tid + (uint32_t)q * kDecThreads;
+            const uint32_t t = tid + (uint32_t)q * nt;
             const uint32_t m = (sb0 + (t >> 8)) * kWave + (t & 63u), jp = (t >> 6) & 3u;
             const uint32_t mc = ((t < SB * 256u) && (m < p.M)) ? m : 0u;     // unconditional loads, clamped index
             E::load_raw2(p.scales, (size_t)8 * mc + 2 * jp, sc0[q], sc1[q]);
@@ -427,7 +449,7 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
         __syncthreads();
 #pragma unroll
         for (int q = 0; q < kMergeTasks; ++q) {
-            const uint32_t t = tid + (uint32_t)q * kDecThreads;
+            const uint32_t t = tid + (uint32_t)q * nt;
             const uint32_t lw = t & 63u, jp = (t >> 6) & 3u, sl = t >> 8;
             const uint32_t m = (sb0 + sl) * kWave + lw;
             if (t >= SB * 256u || m >= p.M) continue;
@@ -468,7 +490,7 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
         const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
         dec_load_x4<DT>(p, lo, len, 4u * tid, xpre);
     }
-    for (uint32_t i = tid; i < p.slots_per_block; i += kDecThreads) lrows[i] = -1;
+    for (uint32_t i = tid; i < p.slots_per_block; i += blockDim.x) lrows[i] = -1;
     uint32_t nslots = 0;
     if (p.fused_select) {
         uint32_t t = 0;
@@ -482,7 +504,7 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
         const uint32_t lo = cgid * per;
         const uint32_t hi = (lo + per) < p.k_total ? (lo + per) : p.k_total;
         __syncthreads();
-        for (uint32_t i = lo + tid; i < hi; i += kDecThreads) {
+        for (uint32_t i = lo + tid; i < hi; i += blockDim.x) {
             const int32_t row = p.sel_rows[i];
             const bool ok = row >= 0 && (uint32_t)row < p.K;       // out-of-range indices are ignored
             lrows[i - lo] = ok ? row : -1;

@@ -381,6 +381,69 @@ def test_selector_edge_cases_general_path(c_oracle):
         ext.destroy_dec_config(cfg)
 
 
+@pytest.mark.parametrize("waves", [4, 7, 8])
+def test_dec_in_smaller_workgroups(waves, c_oracle):
+    """The DEC role in workgroups of 4 to 16 waves: fast selection with few and with many candidates, the
+    general path (non-monotone floors, select-all), caller-supplied indices, short last chunk."""
+    from decdec_amd import _lib
+    _lib.set_option("dec_block_waves", waves)
+    try:
+        for K, N, k_chunk, n_tb in [(4096, 4096, 8, 16), (4096, 1024, 64, 8), (14336, 4096, 20, 24),
+                                    (2048 + 512, 64, 32, 4), (5120, 7680, 32, 32)]:
+            L = make_dec_layer(K, N, seed=K + N + k_chunk)
+            ctx, rows, acts = _ctx(n_tb, K, torch.float16)
+            cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+            out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+            ext.dec(cfg, L["x"].cuda(), out)
+            torch.cuda.synchronize()
+            want_rows, want_acts, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+            k = k_chunk * K // 1024
+            assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k]), (K, N, k_chunk)
+            assert (rows.cpu().numpy()[k:] == -7).all()
+            want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+            assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL, (K, N, k_chunk)
+            # caller-supplied indices
+            topk = torch.topk(L["x"][0, 0].abs().float(), k).indices.to(torch.int32).cuda()
+            rows[:k] = topk
+            out.zero_()
+            ext.unfused_dec(cfg, L["x"].cuda(), out)
+            torch.cuda.synchronize()
+            want = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), topk.cpu().numpy())
+            assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+            ext.destroy_dec_config(cfg)
+        # general path: reversed thresholds, ties, inf / NaN
+        K, N, k_chunk = 3072, 256, 32
+        L = make_dec_layer(K, N, seed=21)
+        x = L["x"].clone()
+        x[0, 0, 5] = float("inf"); x[0, 0, 1030] = float("nan"); x[0, 0, 2050:2200] = 3.0
+        for th in (torch.flip(L["th"], dims=[0]).contiguous(), torch.full_like(L["th"], 2.0), L["th"]):
+            ctx, rows, acts = _ctx(4, K, torch.float16)
+            cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], th)
+            out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+            ext.dec(cfg, x.cuda(), out)
+            torch.cuda.synchronize()
+            want_rows, _, filled = O.select_channels(np_of(x), np_of(th), k_chunk)
+            got = rows.cpu().numpy()[: want_rows.shape[0]]
+            assert np.array_equal(got[filled], want_rows[filled])
+            assert (got[~filled] == -7).all()
+            ext.destroy_dec_config(cfg)
+        # select-all
+        K, N = 2048, 512
+        L = make_dec_layer(K, N, seed=3)
+        ctx, rows, acts = _ctx(8, K, torch.float16)
+        cfg = ext.create_dec_config(ctx, 1024, L["cheat"], L["scales"], L["th"])
+        out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+        ext.dec(cfg, L["x"].cuda(), out)
+        torch.cuda.synchronize()
+        R = F.unpack_residual(L["cheat"], L["scales"]).double()
+        want = (L["x"].double().reshape(1, -1) @ R).reshape(-1).numpy()
+        assert rel_err(np_of(out).reshape(-1), want)[0] <= TOL
+        assert sorted(rows.cpu().numpy()[:K].tolist()) == list(range(K))
+        ext.destroy_dec_config(cfg)
+    finally:
+        _lib.set_option("dec_block_waves", 16)
+
+
 def test_residual_on_device_is_used_in_place(c_oracle, capfd):
     K, N, k_chunk = 4096, 1024, 32
     L = make_dec_layer(K, N, seed=13)
