@@ -12,9 +12,10 @@ the parameters:
   2. fine-grained search (tuner.py:264-312): modules take further +1 steps of k_chunk, cheapest step
      first, while the layer stays within the budget.
 
-`tune()` is pure Python on a timing table and runs anywhere; `measure()` needs the GPU.
+`tune()` is pure Python on a timing table and runs anywhere; `measure()` (isolated launches) and
+`measure_in_model()` (the modules inside the captured decode step, which is what a user will run) need the GPU.
 
-    python -m decdec_amd.autotune --model llama3-8b --algo anyprec --bitwidth 3 --target-slowdown 2.5
+    python -m decdec_amd.autotune --model llama3-8b --algo anyprec --bitwidth 3 --target-slowdown 2.5 [--in-model]
 """
 from __future__ import annotations
 
@@ -176,6 +177,10 @@ def measure(matrix_dims: dict, algo: str, bitwidth: int, n_tb_values, k_chunk_va
             i[0] += 1
             base(i[0] % nb)
         t_base = graph_time(run_base)
+        if not n_tb_values:
+            results[name] = (t_base, {})
+            del ws
+            continue
         rows = torch.zeros(K, dtype=torch.int32, device=dev)
         acts = torch.zeros(K, dtype=torch.float16, device=dev)
         th = F.calibrate_thresholds(K, g, draws=8)
@@ -209,6 +214,63 @@ def measure(matrix_dims: dict, algo: str, bitwidth: int, n_tb_values, k_chunk_va
     return results
 
 
+FULL_NAMES = {"llama3-8b": "Meta-Llama-3-8B-Instruct", "phi3-medium": "Phi-3-medium-4k-instruct",
+              "llama3-70b": "Meta-Llama-3-70B-Instruct"}
+
+
+def measure_in_model(model: str, algo: str, bitwidth: int, n_tb_values, k_chunk_values, group_size: int = 128,
+                     n_layer=None, prompt_len: int = 64, new_tokens: int = 49, log=None):
+    """Times the modules where they run: inside the graph-captured decode step of the random-init model
+    (the reference profiles its decode run, autotuner/run_profile.py:46-56).  For every n_tb and k_chunk, DEC is
+    switched on for ONE module kind at a time; the change of the time per token, divided by the number of layers,
+    is what that module's launch costs over its base GEMV in place.  Returns (results for `tune`, info) with
+    info = {"token_us_base", "n_layer", "model", "evaluate": callable(k_chunks, n_tb) -> us per token}."""
+    import torch
+    from . import generate as G
+    m = G.build_model(FULL_NAMES[model], algo, bitwidth, group_size, n_layer=n_layer)
+    gen = torch.Generator().manual_seed(3)
+    prompt = torch.randint(0, m.config.vocab_size, (prompt_len,), generator=gen).cuda()
+    cache = max(256, prompt_len + new_tokens)
+
+    def token_us():
+        best = float("inf")
+        for _ in range(2):
+            _, dt = G.generate(m, prompt, new_tokens, True, cache)
+            best = min(best, dt / (new_tokens - 1) * 1e6)
+        return best
+
+    t_base = token_us()
+    m.load_dec_data(G.random_dec_data(m, G.calibrate_thresholds(m, seq_len=min(256, cache))))
+    dims = MODELS[model]
+    k_max = max(k_chunk_values)
+    names = list(dims)
+    base = measure(dims, algo, bitwidth, [], [], group_size)            # isolated base GEMV times
+    tables = {name: {} for name in names}
+    first = True
+    for n_tb in n_tb_values:
+        if first:
+            m.create_dec_context(n_tb, buffer_size=max(1024, k_max * (m.config.intermediate_size // 1024 + 1)))
+            m.set_dec_config([0, 0, 0, 0])                              # pins the residuals once
+            first = False
+        else:
+            m.update_dec_context(n_tb)
+        for i, name in enumerate(names):
+            tables[name][n_tb] = {}
+            for k in k_chunk_values:
+                m.update_dec_config([k if j == i else 0 for j in range(4)])
+                tables[name][n_tb][k] = base[name][0] + (token_us() - t_base) / m.config.n_layer
+            if log:
+                log(f"{name} base {base[name][0]:.2f} us, in-model, n_tb {n_tb}: " +
+                    " ".join(f"k{k}={t:.2f}" for k, t in tables[name][n_tb].items()))
+
+    def evaluate(k_chunks, n_tb):
+        m.update_dec_context(n_tb)
+        m.update_dec_config(list(k_chunks))
+        return token_us()
+    results = {name: (base[name][0], tables[name]) for name in names}
+    return results, {"token_us_base": t_base, "n_layer": m.config.n_layer, "model": FULL_NAMES[model], "evaluate": evaluate}
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--model", choices=sorted(MODELS), default="llama3-8b")
@@ -219,6 +281,9 @@ def main(argv=None):
     ap.add_argument("--max-n-tb", type=int, default=32)
     ap.add_argument("--n-tb-step", type=int, default=4)
     ap.add_argument("--max-k-chunk", type=int, default=0, help="0: twice the break-even estimate, at least 8")
+    ap.add_argument("--in-model", action="store_true",
+                    help="time the modules inside the graph-captured decode step of the random-init model")
+    ap.add_argument("--n-layer", type=int, default=None, help="--in-model: build fewer layers than the model has")
     args = ap.parse_args(argv)
     dims = MODELS[args.model]
     k_max = args.max_k_chunk or max(8, 2 * k_chunk_estimate(args.bitwidth))
@@ -226,9 +291,21 @@ def main(argv=None):
     ks = list(range(1, k_max + 1))
     print(f"break-even k_chunk estimate {k_chunk_estimate(args.bitwidth)}; sweeping k_chunk 1..{k_max}, n_tb {n_tbs}",
           file=sys.stderr)
-    res = measure(dims, args.algo, args.bitwidth, n_tbs, ks, log=lambda s: print(s, file=sys.stderr, flush=True))
+    log = lambda s: print(s, file=sys.stderr, flush=True)
+    if args.in_model:
+        res, info = measure_in_model(args.model, args.algo, args.bitwidth, n_tbs, ks, n_layer=args.n_layer, log=log)
+    else:
+        res, info = measure(dims, args.algo, args.bitwidth, n_tbs, ks, log=log), None
     out = tune(res, 1 + args.target_slowdown / 100, dims)
     out["target_slowdown_pct"] = args.target_slowdown
+    if info is not None:
+        out["measured"] = "in the captured decode step"
+        out["token_us_base"] = round(info["token_us_base"], 1)
+        out["predicted_token_slowdown_pct"] = round(
+            (out["layer_time"] - out["layer_baseline"]) * info["n_layer"] / info["token_us_base"] * 100, 2)
+        if out["best_max_n_tb"] is not None:
+            t = info["evaluate"](out["k_chunk_per_module"], out["best_max_n_tb"])
+            out["measured_token_slowdown_pct"] = round((t / info["token_us_base"] - 1) * 100, 2)
     print(json.dumps(out))
 
 

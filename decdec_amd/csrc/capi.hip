@@ -54,13 +54,13 @@ struct Options {
     int sqllm_ktiles = 0;
     int dec_trace = 0;
     int anyprec_rg = 0;
-    int dec_block_waves = 16;   // waves of a standalone DEC workgroup (4 .. 16)
+    int dec_block_waves = 16;   // waves of a standalone DEC workgroup: 4, 8 or 16
     int fused_two_per_cu = -1;  // fused launches: 1 / 0 = always / never two workgroups per compute unit, -1 = by estimate
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
 uint32_t dec_block_threads() {
-    const int w = std::min(std::max(g_opt.dec_block_waves, (int)kMinDecWaves), (int)kDecWaves);
+    const int w = g_opt.dec_block_waves <= 4 ? 4 : (g_opt.dec_block_waves <= 8 ? 8 : 16);
     return (uint32_t)w * kWave;
 }
 

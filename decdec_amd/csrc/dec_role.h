@@ -63,40 +63,36 @@ __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves 
 // General path: every wave tests its 64 channels against all 32 buckets (one ballot per bucket),
 // per-(bucket, wave) counts are prefix-summed, and each member computes its position.  Exact for any
 // floors (non-monotone floors can put a channel into several buckets, as in the reference kernel).
-template <int DT>
+template <int DT, int NW>
 __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t c, uint32_t t_local, uint32_t kc,
                                                 int32_t* lrows, float* lacts, uint32_t* cnt, uint32_t* pre,
                                                 bool write_global) {
     using E = Elem<DT>;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    constexpr uint32_t nw = NW;
     const uint32_t lo = c * kChunk;
     const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
-    // The chunk is 16 groups of 64 channels; wave w plays groups w, w + nw, ... (one group per wave in a
+    // The chunk is 16 groups of 64 channels; wave w takes groups w, w + nw, ... (one group per wave in a
     // 1024-thread workgroup, four in a 256-thread one).
-    constexpr int kPasses = kChunk / kWave / kMinDecWaves;
+    // Nothing is kept between the counting and the placing step but the counts: a group's activations are
+    // read again and its memberships recomputed (this path is rare; registers held here would be charged to
+    // every launch of the kernels that contain it).
+    const uint32_t ngroups = (uint32_t)(kChunk / kWave);
     const float myfloor = p.floors[lane & 31u];                      // lane i holds floor[i]
-    float xv[kPasses];
-    uint32_t member[kPasses];
-#pragma unroll
-    for (int ps = 0; ps < kPasses; ++ps) {
-        const uint32_t vw = (uint32_t)ps * nw + wave;                // group of this pass
-        member[ps] = 0;
-        xv[ps] = 0.f;
-        if (vw < (uint32_t)(kChunk / kWave)) {                       // uniform per wave
-            const uint32_t ch = vw * kWave + lane;
-            const bool in = ch < len;
-            xv[ps] = in ? E::load(p.x, lo + ch) : 0.f;
-            const float a = in ? __builtin_fabsf(xv[ps]) : __builtin_nanf("");   // NaN is a member of no bucket
-            float ce = __builtin_inff();
 #pragma unroll 1
-            for (int i = 0; i < kBuckets; ++i) {
-                const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
-                const bool bit = (a >= fl) && (a < ce);
-                ce = fl;
-                member[ps] |= (uint32_t)bit << i;
-                const unsigned long long m = __ballot(bit);
-                if (lane == 0) cnt[i * 16 + vw] = (uint32_t)__popcll(m);
-            }
+    for (uint32_t vw = wave; vw < ngroups; vw += nw) {
+        const uint32_t ch = vw * kWave + lane;
+        const bool in = ch < len;
+        const float xv = in ? E::load(p.x, lo + ch) : 0.f;
+        const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");   // NaN is a member of no bucket
+        float ce = __builtin_inff();
+#pragma unroll 1
+        for (int i = 0; i < kBuckets; ++i) {
+            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+            const bool bit = (a >= fl) && (a < ce);
+            ce = fl;
+            const unsigned long long m = __ballot(bit);
+            if (lane == 0) cnt[i * 16 + vw] = (uint32_t)__popcll(m);
         }
     }
     __syncthreads();
@@ -115,25 +111,29 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
         for (int q = 0; q < 8; ++q) { pre[lane * 8 + q] = run; run += v[q]; }
     }
     __syncthreads();
-#pragma unroll
-    for (int ps = 0; ps < kPasses; ++ps) {
-        const uint32_t vw = (uint32_t)ps * nw + wave;
-        if (vw >= (uint32_t)(kChunk / kWave)) continue;              // uniform per wave
+#pragma unroll 1
+    for (uint32_t vw = wave; vw < ngroups; vw += nw) {
         const uint32_t ch = vw * kWave + lane;
+        const bool in = ch < len;
+        const float xv = in ? E::load(p.x, lo + ch) : 0.f;
+        const float a = in ? __builtin_fabsf(xv) : __builtin_nanf("");
+        float ce = __builtin_inff();
 #pragma unroll 1
         for (int i = 0; i < kBuckets; ++i) {
             if (pre[i * 16] >= kc) break;                            // uniform: later buckets start even later
-            const bool bit = (member[ps] >> i) & 1u;
+            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+            const bool bit = (a >= fl) && (a < ce);
+            ce = fl;
             const unsigned long long m = __ballot(bit);
             if (bit) {
                 const uint32_t pos = pre[i * 16 + vw] + ballot_rank(m);
                 if (pos < kc) {
                     const uint32_t slot = t_local * p.k_chunk + pos;
                     lrows[slot] = (int32_t)(lo + ch);
-                    lacts[slot] = xv[ps];
+                    lacts[slot] = xv;
                     if (write_global) {
                         p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)(lo + ch);
-                        E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xv[ps]);
+                        E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xv);
                     }
                 }
             }
@@ -179,7 +179,7 @@ __device__ __forceinline__ void dec_load_x4(const DecParams& p, uint32_t lo, uin
     for (int s = 0; s < 4; ++s) xr[s] = Elem<DT>::load_raw(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
 }
 
-template <int DT>
+template <int DT, int NW>
 __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
                                                  int32_t* lrows, float* lacts, uint32_t* cnt,
                                                  uint32_t* pre, float* red, bool write_global,
@@ -264,7 +264,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     const u32x2 hd = *(const u32x2*)hdr;
     if (hd[0] == 0u) {                                     // uniform
         __syncthreads();                                   // hdr is read before cnt is reused
-        dec_select_general<DT>(p, c, t_local, kc, lrows, lacts, cnt, pre, write_global);
+        dec_select_general<DT, NW>(p, c, t_local, kc, lrows, lacts, cnt, pre, write_global);
         return;
     }
     const uint32_t total = hd[1];
@@ -327,7 +327,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per wave and round
         const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
 #pragma unroll 1
-        for (uint32_t tile = wave; tile < ntiles; tile += (blockDim.x >> 6)) {
+        for (uint32_t tile = wave; tile < ntiles; tile += (uint32_t)NW) {
             const uint32_t jg = tile % njg, iq = tile / njg;
             const uint32_t j = jg * 64u + lane;
             const uint32_t mykey = j < total ? key[j] : 0u;
@@ -376,12 +376,13 @@ __device__ __forceinline__ void dec_accumulate_word(uint32_t w, float act, float
     acc[7] += (float)(hi >> 24) * act;
 }
 
-template <int DT>
+template <int DT, int NW>
 __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint32_t sgid, uint32_t nslots,
                                           const int32_t* lrows, const float* lacts, float* red) {
     using E = Elem<DT>;
     constexpr int U = 8;                                // residual rows in flight per wave
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6, nt = blockDim.x;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    constexpr uint32_t nw = NW, nt = NW * kWave;
     const uint32_t seg_lo = sgid * p.segs_per_block;
     const uint32_t seg_hi = (seg_lo + p.segs_per_block) < p.nseg ? (seg_lo + p.segs_per_block) : p.nseg;
 
@@ -469,7 +470,7 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
 }
 
 // ---- the role -------------------------------------------------------------------------------------
-template <int DT>
+template <int DT, int NW = kDecWaves>
 __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsigned char* smem) {
     using E = Elem<DT>;
     const uint32_t tid = threadIdx.x;
@@ -490,13 +491,13 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
         const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
         dec_load_x4<DT>(p, lo, len, 4u * tid, xpre);
     }
-    for (uint32_t i = tid; i < p.slots_per_block; i += blockDim.x) lrows[i] = -1;
+    for (uint32_t i = tid; i < p.slots_per_block; i += (uint32_t)NW * kWave) lrows[i] = -1;
     uint32_t nslots = 0;
     if (p.fused_select) {
         uint32_t t = 0;
         for (uint32_t c = cgid; c < p.num_chunks; c += p.cg, ++t) {
             __syncthreads();      // list initialised; cnt/pre of the previous chunk no longer read
-            dec_select_chunk<DT>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0, have_xpre && t == 0, xpre);
+            dec_select_chunk<DT, NW>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0, have_xpre && t == 0, xpre);
         }
         nslots = t * p.k_chunk;
     } else {
@@ -504,7 +505,7 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
         const uint32_t lo = cgid * per;
         const uint32_t hi = (lo + per) < p.k_total ? (lo + per) : p.k_total;
         __syncthreads();
-        for (uint32_t i = lo + tid; i < hi; i += blockDim.x) {
+        for (uint32_t i = lo + tid; i < hi; i += (uint32_t)NW * kWave) {
             const int32_t row = p.sel_rows[i];
             const bool ok = row >= 0 && (uint32_t)row < p.K;       // out-of-range indices are ignored
             lrows[i - lo] = ok ? row : -1;
@@ -514,7 +515,7 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
     }
     __syncthreads();
     dec_stamp(p, bid, 1);
-    dec_fetch<DT>(p, bid, sgid, nslots, lrows, lacts, red);
+    dec_fetch<DT, NW>(p, bid, sgid, nslots, lrows, lacts, red);
     dec_stamp(p, bid, 4);
 }
 

@@ -3,20 +3,32 @@
 
 namespace decdec {
 
-template <int DT>
-__global__ __launch_bounds__(kDecThreads) void dec_kernel(const DecParams p) {
+// NW = waves of the workgroup (16 by default; 4 and 8 exist for callers that want DEC workgroups which hold
+// a smaller share of a compute unit).
+template <int DT, int NW>
+__global__ __launch_bounds__(NW * kWave) void dec_kernel(const DecParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    dec_role<DT>(p, blockIdx.x, smem);
+    dec_role<DT, NW>(p, blockIdx.x, smem);
 }
 
-hipError_t launch_dec(int dt, const DecParams& p, const LaunchDims& d, hipStream_t s) {
+template <int NW>
+static hipError_t launch_dec_nw(int dt, const DecParams& p, const LaunchDims& d, hipStream_t s) {
     switch (dt) {
-        case kFP32: hipLaunchKernelGGL(dec_kernel<kFP32>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
-        case kFP16: hipLaunchKernelGGL(dec_kernel<kFP16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
-        case kBF16: hipLaunchKernelGGL(dec_kernel<kBF16>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
+        case kFP32: hipLaunchKernelGGL((dec_kernel<kFP32, NW>), dim3(d.grid), dim3(NW * kWave), d.lds, s, p); break;
+        case kFP16: hipLaunchKernelGGL((dec_kernel<kFP16, NW>), dim3(d.grid), dim3(NW * kWave), d.lds, s, p); break;
+        case kBF16: hipLaunchKernelGGL((dec_kernel<kBF16, NW>), dim3(d.grid), dim3(NW * kWave), d.lds, s, p); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
+}
+
+hipError_t launch_dec(int dt, const DecParams& p, const LaunchDims& d, hipStream_t s) {
+    switch (d.block / kWave) {
+        case 4: return launch_dec_nw<4>(dt, p, d, s);
+        case 8: return launch_dec_nw<8>(dt, p, d, s);
+        case 16: return launch_dec_nw<16>(dt, p, d, s);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 // Pure-ALU spin that keeps `blocks` workgroups of 1024 threads resident (the counterpart of the

@@ -78,3 +78,20 @@ def test_invalid_handles_and_arguments_fail_cleanly():
     assert lib.decdec_sqllm_gemv(p, p, p, p, 5, 1, 1024, 8, None) != 0 and "Bitwidth must be 3 or 4" in _lib.last_error()
     assert lib.decdec_lutgemm_gemv(p, p, p, p, p, 9, 128, 1, 1024, 8, None) != 0 and "between 1 and 8" in _lib.last_error()
     assert lib.decdec_lutgemm_gemv(p, p, p, p, p, 3, 48, 1, 1024, 8, None) != 0 and "group_size" in _lib.last_error()
+
+
+def test_kernel_register_budgets():
+    """The launch logic counts on register budgets (two 1024-thread workgroups per compute unit for the budgeted
+    fused instances, no scratch in the decode-path kernels); the build records what the compiler reports."""
+    import json
+    from decdec_amd import build
+    if not os.path.exists(build.RESOURCES_PATH):
+        pytest.skip("library was not built in this tree")
+    kernels = json.load(open(build.RESOURCES_PATH))
+    assert len(kernels) > 40 and any("dec_sqllm_kernel" in k for k in kernels)
+    assert build.check_resources(kernels) == []
+    # the checker does flag what it is meant to flag
+    broken = {"_ZN6decdec16dec_sqllm_kernelILi1ELb1EEEvNS_9DecParamsEjNS_11SqllmParamsE":
+              {"occupancy": 8, "scratch": 68, "sgprs": 78, "vgprs": 64}}
+    assert len(build.check_resources(broken)) >= 1
+

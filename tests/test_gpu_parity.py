@@ -381,9 +381,9 @@ def test_selector_edge_cases_general_path(c_oracle):
         ext.destroy_dec_config(cfg)
 
 
-@pytest.mark.parametrize("waves", [4, 7, 8])
+@pytest.mark.parametrize("waves", [4, 8])
 def test_dec_in_smaller_workgroups(waves, c_oracle):
-    """The DEC role in workgroups of 4 to 16 waves: fast selection with few and with many candidates, the
+    """The DEC role in workgroups of 4 and 8 waves: fast selection with few and with many candidates, the
     general path (non-monotone floors, select-all), caller-supplied indices, short last chunk."""
     from decdec_amd import _lib
     _lib.set_option("dec_block_waves", waves)
