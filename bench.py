@@ -196,13 +196,16 @@ def kernels_leg(torch, ext, F):
 
     rows_out = []
     cases = []
-    for K, N in [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (8192, 8192), (8192, 28672), (28672, 8192)]:
-        cases.append(("anyprec3", K, N))
-    for K, N in [(5120, 7680), (5120, 5120), (5120, 35840), (17920, 5120)]:
-        cases.append(("lutgemm3g128", K, N))
+    n_tb = 32
+    for K, N in [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)]:            # Llama-3-8B
+        cases.append(("anyprec3", K, N, (32,)))
+    for K, N in [(8192, 8192), (8192, 1024), (8192, 28672), (28672, 8192)]:            # Llama-3-70B: k_chunk 16 and 32
+        cases.append(("anyprec3", K, N, (16, 32)))
+    for K, N in [(5120, 7680), (5120, 5120), (5120, 35840), (17920, 5120)]:            # Phi-3-medium
+        cases.append(("lutgemm3g128", K, N, (32,)))
     for K, N in [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096)]:
-        cases.append(("sqllm4", K, N))
-    for kind, K, N in cases:
+        cases.append(("sqllm4", K, N, (32,)))
+    for kind, K, N, k_chunks in cases:
         x = F.make_activation(K, g).to(dev)
         out = torch.zeros(1, 1, N, device=dev, dtype=torch.float16)
         if kind == "anyprec3":
@@ -233,19 +236,23 @@ def kernels_leg(torch, ext, F):
             i[0] += 1
             base(i[0] % nb)
         tb = graph_time(run_base)
-        keep, cfg = dec_cfg(K, N, 32, 8)
+        keep, cfg = dec_cfg(K, N, k_chunks[0], n_tb)
+        for kc in k_chunks:
+            if kc != k_chunks[0]:
+                ext.update_dec_config(cfg, keep[3], kc)
 
-        def run_fused():
-            i[0] += 1
-            fused(cfg, i[0] % nb)
-        tf = graph_time(run_fused, reps=10, iters=10)
-        td = graph_time(lambda: ext.dec(cfg, x, out), reps=10, iters=10)
-        hb = 32 * K // 1024 * N // 2
-        rows_out.append({"kernel": kind, "K": K, "N": N, "base_us": round(tb, 2), "base_gbs": round(by / tb / 1e3, 1),
-                         "base_frac_hbm": round(by / tb / 1e3 / HBM_PEAK_GBS, 3), "dec_us": round(td, 2),
-                         "dec_host_gbs": round(hb / td / 1e3, 1), "dec_frac_link": round(hb / td / 1e3 / 64.0, 3),
-                         "fused_us": round(tf, 2), "slowdown_pct": round((tf / tb - 1) * 100, 1)})
-        print(json.dumps(rows_out[-1]), file=sys.stderr, flush=True)
+            def run_fused():
+                i[0] += 1
+                fused(cfg, i[0] % nb)
+            tf = graph_time(run_fused, reps=10, iters=10)
+            td = graph_time(lambda: ext.dec(cfg, x, out), reps=10, iters=10)
+            hb = kc * K // 1024 * N // 2
+            rows_out.append({"kernel": kind, "K": K, "N": N, "k_chunk": kc, "n_tb": n_tb, "base_us": round(tb, 2),
+                             "base_gbs": round(by / tb / 1e3, 1), "base_frac_hbm": round(by / tb / 1e3 / HBM_PEAK_GBS, 3),
+                             "dec_us": round(td, 2), "dec_host_gbs": round(hb / td / 1e3, 1),
+                             "dec_frac_link": round(hb / td / 1e3 / 64.0, 3), "fused_us": round(tf, 2),
+                             "slowdown_pct": round((tf / tb - 1) * 100, 1)})
+            print(json.dumps(rows_out[-1]), file=sys.stderr, flush=True)
         ext.destroy_dec_config(cfg)
         ext.destroy_dec_context(keep[3])
         del ws
