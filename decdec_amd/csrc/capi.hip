@@ -891,4 +891,16 @@ int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void*
     return kOk;
 }
 
+int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out, int dtype,
+                       uint32_t rows, uint32_t dim, float eps, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(x && weight && normed_out, "null pointer argument");
+    DD_CHECK(dim >= 4 && dim % 4 == 0 && dim <= 16384, "dim must be a multiple of 4 up to 16384, got %u", dim);
+    DD_CHECK(((uintptr_t)x % 8) == 0 && ((uintptr_t)weight % 8) == 0 && ((uintptr_t)normed_out % 8) == 0 &&
+             ((uintptr_t)y % 8) == 0 && ((uintptr_t)h_out % 8) == 0, "tensors must be 8-byte aligned");
+    if (rows == 0) return kOk;
+    DD_HIP(launch_add_rmsnorm(dtype, x, y, weight, h_out, normed_out, rows, dim, eps, (hipStream_t)stream));
+    return kOk;
+}
+
 }  // extern "C"

@@ -32,6 +32,7 @@ template <> struct Elem<kFP32> {
     // storage bits of element i, and their value (lets a caller request a value long before it converts it)
     static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint32_t*)p)[i]; }
     static __device__ __forceinline__ float from_raw(uint32_t r) { return __uint_as_float(r); }
+    static __device__ __forceinline__ uint32_t to_raw(float f) { return __float_as_uint(f); }
     // storage bits of the even-aligned pair (i, i + 1) and their values
     static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
         const u32x2 v = *(const u32x2*)((const uint32_t*)p + i); a = v[0]; b = v[1];
@@ -81,6 +82,9 @@ template <> struct Elem<kFP16> {
     static __device__ __forceinline__ float from_raw(uint32_t r) {
         const uint16_t h = (uint16_t)r; _Float16 v; __builtin_memcpy(&v, &h, 2); return (float)v;
     }
+    static __device__ __forceinline__ uint32_t to_raw(float f) {
+        const _Float16 v = (_Float16)f; uint16_t h; __builtin_memcpy(&h, &v, 2); return h;
+    }
     static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
         a = *(const uint32_t*)((const uint16_t*)p + i); b = 0u;
     }
@@ -105,6 +109,7 @@ template <> struct Elem<kBF16> {
     static __device__ __forceinline__ float load(const void* p, size_t i) { return bf16_bits_to_f32(((const uint16_t*)p)[i]); }
     static __device__ __forceinline__ uint32_t load_raw(const void* p, size_t i) { return ((const uint16_t*)p)[i]; }
     static __device__ __forceinline__ float from_raw(uint32_t r) { return bf16_bits_to_f32((uint16_t)r); }
+    static __device__ __forceinline__ uint32_t to_raw(float f) { return f32_to_bf16_bits(f); }
     static __device__ __forceinline__ void load_raw2(const void* p, size_t i, uint32_t& a, uint32_t& b) {
         a = *(const uint32_t*)((const uint16_t*)p + i); b = 0u;
     }

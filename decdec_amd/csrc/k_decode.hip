@@ -127,6 +127,94 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ 
     E::store(out, i, a / (1.f + __expf(-a)) * b);
 }
 
+// h = x + y (skipped when y is null), normed = h / rms(h) * weight: the residual add and the RMS normalisation that
+// follows it in a decoder block.  One workgroup per row, four neighbouring elements per thread and pass (one 8-byte
+// load each of x, y and the weight, all requested before anything is used), statistics in fp32.
+template <int DT, int PASSES>
+__global__ __launch_bounds__(1024) void add_rmsnorm_kernel(const void* __restrict__ x, const void* __restrict__ y,
+                                                           const void* __restrict__ weight, void* __restrict__ h_out,
+                                                           void* __restrict__ normed_out, uint32_t dim, float eps) {
+    using E = Elem<DT>;
+    __shared__ float wsum[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, nw = blockDim.x >> 6;
+    const size_t row = (size_t)blockIdx.x * dim;
+    const bool have_y = y != nullptr;
+    u32x2 xr[PASSES], yr[PASSES], wr[PASSES];
+#pragma unroll
+    for (int k = 0; k < PASSES; ++k) {
+        const uint32_t i = 4u * (tid + (uint32_t)k * blockDim.x);
+        const uint32_t ic = (i + 4u <= dim) ? i : 0u;       // groups past the end re-read the first one; never used
+        xr[k] = *(const u32x2*)((const uint16_t*)x + row + ic);
+        yr[k] = have_y ? *(const u32x2*)((const uint16_t*)y + row + ic) : u32x2{0u, 0u};
+        wr[k] = *(const u32x2*)((const uint16_t*)weight + ic);
+    }
+    float v[PASSES][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < PASSES; ++k) {
+        const uint32_t i = 4u * (tid + (uint32_t)k * blockDim.x);
+        const bool ok = i + 4u <= dim;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t sh = (e & 1) ? 16u : 0u;
+            float a = E::from_raw((xr[k][e >> 1] >> sh) & 0xFFFFu);
+            if (have_y) a = E::from_raw(E::to_raw(a + E::from_raw((yr[k][e >> 1] >> sh) & 0xFFFFu)));   // as stored
+            v[k][e] = ok ? a : 0.f;
+            ss += v[k][e] * v[k][e];
+        }
+        if (ok && have_y && h_out != nullptr) {
+            u32x2 o;
+            o[0] = E::to_raw(v[k][0]) | (E::to_raw(v[k][1]) << 16);
+            o[1] = E::to_raw(v[k][2]) | (E::to_raw(v[k][3]) << 16);
+            *(u32x2*)((uint16_t*)h_out + row + i) = o;
+        }
+    }
+    ss = wave_sum_dpp(ss);                                  // total in lane 63
+    if (lane == 63) wsum[wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+    for (uint32_t w = 0; w < nw; ++w) tot += wsum[w];
+    const float r = __builtin_amdgcn_rsqf(tot / (float)dim + eps);
+#pragma unroll
+    for (int k = 0; k < PASSES; ++k) {
+        const uint32_t i = 4u * (tid + (uint32_t)k * blockDim.x);
+        if (i + 4u <= dim) {
+            float o4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o4[e] = v[k][e] * r * E::from_raw((wr[k][e >> 1] >> ((e & 1) ? 16u : 0u)) & 0xFFFFu);
+            u32x2 o;
+            o[0] = E::to_raw(o4[0]) | (E::to_raw(o4[1]) << 16);
+            o[1] = E::to_raw(o4[2]) | (E::to_raw(o4[3]) << 16);
+            *(u32x2*)((uint16_t*)normed_out + row + i) = o;
+        }
+    }
+}
+
+template <int DT>
+static hipError_t launch_add_rmsnorm_dt(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
+                                        uint32_t rows, uint32_t dim, float eps, hipStream_t s) {
+    const uint32_t groups = dim / 4u;
+    uint32_t threads = 64;
+    while (threads < 1024 && threads < groups) threads *= 2;
+    const dim3 grid(rows), block(threads);
+    if (groups <= threads)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<DT, 1>), grid, block, 0, s, x, y, weight, h_out, normed_out, dim, eps);
+    else if (groups <= 2 * threads)
+        hipLaunchKernelGGL((add_rmsnorm_kernel<DT, 2>), grid, block, 0, s, x, y, weight, h_out, normed_out, dim, eps);
+    else
+        hipLaunchKernelGGL((add_rmsnorm_kernel<DT, 4>), grid, block, 0, s, x, y, weight, h_out, normed_out, dim, eps);
+    return hipGetLastError();
+}
+
+hipError_t launch_add_rmsnorm(int dt, const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
+                              uint32_t rows, uint32_t dim, float eps, hipStream_t s) {
+    if (dim % 4u != 0 || dim > 16384u) return hipErrorInvalidValue;
+    if (dt == kFP16) return launch_add_rmsnorm_dt<kFP16>(x, y, weight, h_out, normed_out, rows, dim, eps, s);
+    if (dt == kBF16) return launch_add_rmsnorm_dt<kBF16>(x, y, weight, h_out, normed_out, rows, dim, eps, s);
+    return hipErrorInvalidValue;
+}
+
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s) {
     const uint32_t threads = (p.n_head + p.n_kv) * (p.head_dim / 2) + p.n_kv * p.head_dim;
     const dim3 grid((threads + 255) / 256), block(256);

@@ -43,3 +43,17 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _half_cuda(gate_up, out)
     _check(gate_up.numel() == 2 * out.numel(), "gate_up must hold twice as many elements as out")
     _lib.check(_lib.load().decdec_silu_mul(_ptr(gate_up), _ptr(out), _dt(out), out.numel(), _stream()))
+
+
+def add_rmsnorm(x: torch.Tensor, y, weight: torch.Tensor, h_out, normed_out: torch.Tensor, eps: float) -> None:
+    """Rows of x [..., dim]: h = x + y (written to h_out; y = h_out = None: h = x), normed_out = rmsnorm(h) * weight."""
+    ts = [t for t in (x, y, weight, h_out, normed_out) if t is not None]
+    _half_cuda(*ts)
+    dim = x.shape[-1]
+    _check(weight.numel() == dim and normed_out.shape == x.shape, "weight / normed_out shape mismatch")
+    _check((y is None) == (h_out is None) and (y is None or (y.shape == x.shape and h_out.shape == x.shape)),
+           "y and h_out go together and have the shape of x")
+    _lib.check(_lib.load().decdec_add_rmsnorm(_ptr(x), _ptr(y) if y is not None else None, _ptr(weight),
+                                              _ptr(h_out) if h_out is not None else None, _ptr(normed_out), _dt(x),
+                                              x.numel() // dim, dim, float(eps), _stream()))
+

@@ -6,7 +6,8 @@ Counterpart of the reference's end-to-end/model.py (a gpt-fast style Llama / Phi
 reference's meaning (k_chunks = [qkv, o, gate_up, down]).  Everything that is not a linear layer is
 plain torch: this file exists to drive the linear-layer hot path from a real decode step, not to be a
 model zoo.  A decode step touches only static buffers, so it can be captured in a HIP graph; on the GPU
-its rotary embedding, cache append, attention and gated activation run on the library's helper kernels
+its residual adds + normalisations, rotary embedding, cache append, attention and gated activation run on the library's
+helper kernels
 (``decode_ops``), a prefill or CPU pass on torch ops.
 """
 from __future__ import annotations
@@ -176,6 +177,23 @@ class TransformerBlock(nn.Module):
         h = x + self.attention(self.input_layernorm(x), mask, cos, sin, input_pos, rope_tables_full)
         return h + self.feed_forward(self.post_attention_layernorm(h), rope_tables_full is not None)
 
+    def decode_step(self, h, branch, input_pos, rope_tables_full):
+        """One token on the helper kernels.  `h` is the residual stream before this block, `branch` the output of
+        the previous block's feed-forward that has not been added yet (None for the first block); returns the
+        stream after this block's attention and this block's feed-forward output, again not yet added."""
+        from . import decode_ops
+        n1 = torch.empty_like(h)
+        if branch is None:
+            decode_ops.add_rmsnorm(h, None, self.input_layernorm.weight, None, n1, self.input_layernorm.eps)
+            h0 = h
+        else:
+            h0 = torch.empty_like(h)
+            decode_ops.add_rmsnorm(h, branch, self.input_layernorm.weight, h0, n1, self.input_layernorm.eps)
+        a = self.attention(n1, None, None, None, input_pos, rope_tables_full)
+        h1, n2 = torch.empty_like(h), torch.empty_like(h)
+        decode_ops.add_rmsnorm(h0, a, self.post_attention_layernorm.weight, h1, n2, self.post_attention_layernorm.eps)
+        return h1, self.feed_forward(n2, True)
+
     def dec_linears(self):
         """The four compensated linears in the order of the k_chunk lists: qkv, o, gate_up, down."""
         return [self.attention.wqkv, self.attention.wo, self.feed_forward.w1w3, self.feed_forward.w2]
@@ -241,10 +259,14 @@ class Transformer(nn.Module):
             self.output_arena.zero_()
         x = self.tok_embeddings(idx)
         if self.decode_kernels and idx.shape == (1, 1) and x.is_cuda:
+            from . import decode_ops
             full = (self.rope_cos, self.rope_sin)
+            h, branch = x.contiguous(), None
             for layer in self.layers:
-                x = layer(x, None, None, None, input_pos, full)
-            return self.output(self.norm(x))
+                h, branch = layer.decode_step(h, branch, input_pos, full)
+            n = torch.empty_like(h)
+            decode_ops.add_rmsnorm(h, branch, self.norm.weight, torch.empty_like(h), n, self.norm.eps)
+            return self.output(n)
         mask = self.causal_mask.index_select(0, input_pos)                     # [S, max_seq]
         cos, sin = self.rope_cos.index_select(0, input_pos), self.rope_sin.index_select(0, input_pos)
         for layer in self.layers:

@@ -155,7 +155,9 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     ([n_kv_head][max_seq][head_dim]).  A position outside [0, max_seq) writes nothing.
  *   decdec_decode_attention: out[h] = softmax(q[h] . K[kv(h)][0..pos] / sqrt(head_dim)) V[kv(h)][0..pos],
  *     head_dim 64 or 128, grouped-query heads (kv(h) = h / (n_head / n_kv_head)).
- *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n. */
+ *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n.
+ *   decdec_add_rmsnorm: per row of `dim` elements (a multiple of 4, <= 16384; 8-byte aligned tensors), h = x + y rounded to the storage type and written to
+ *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight. */
 int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void* sin_table,
                              const int64_t* pos_device, void* q_out, void* k_cache, void* v_cache,
                              int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
@@ -164,6 +166,8 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
                             const int64_t* pos_device, void* out, int dtype, uint32_t n_head,
                             uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream);
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
+int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
+                       int dtype, uint32_t rows, uint32_t dim, float eps, void* stream);
 
 /* Diagnostics: with option "dec_trace" = 1 every DEC workgroup stores shader-clock stamps of its
  * phases (0 start, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a

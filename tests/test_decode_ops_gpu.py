@@ -76,6 +76,26 @@ def test_silu_mul(n):
     assert _close(out, want, 2e-3)
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (1, 512), (3, 5120), (2, 8192), (1, 68), (2, 14336)])
+def test_add_rmsnorm(rows, dim, dt):
+    g = torch.Generator(device="cuda").manual_seed(2)
+    x = torch.randn(rows, dim, generator=g, device="cuda").to(dt)
+    y = (torch.randn(rows, dim, generator=g, device="cuda") * 0.5).to(dt)
+    w = (1 + 0.1 * torch.randn(dim, generator=g, device="cuda")).to(dt)
+    h, n = torch.empty_like(x), torch.empty_like(x)
+    D.add_rmsnorm(x, y, w, h, n, 1e-5)
+    want_h = (x.float() + y.float()).to(dt)
+    assert torch.equal(h, want_h)
+    hf = want_h.float()
+    want_n = hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + 1e-5) * w.float()
+    assert _close(n, want_n, 2e-2 if dt == torch.bfloat16 else 3e-3)
+    n2 = torch.empty_like(x)
+    D.add_rmsnorm(x, None, w, None, n2, 1e-5)
+    xf = x.float()
+    assert _close(n2, xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5) * w.float(), 2e-2 if dt == torch.bfloat16 else 3e-3)
+
+
 def test_argument_checks():
     a = torch.zeros(8, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError, match="twice as many"):
