@@ -50,54 +50,77 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-// One workgroup per query head.  A group of D/8 lanes owns a cache position (16 bytes of K and of V per
-// lane); a wave visits 64 / (D/8) positions per step, the 16 waves interleave, every group keeps its own
-// running maximum / sum / output (online softmax), and the groups are merged through LDS at the end.
+// `nsplit` workgroups per query head share the positions 0 .. pos (contiguous ranges).  In a workgroup, a group of
+// D/8 lanes owns a cache position (16 bytes of K and of V per lane); a wave visits 64 / (D/8) positions per step
+// and four steps per loop trip (their rows requested together), the 16 waves interleave, every lane group keeps
+// its own running maximum / sum / output (online softmax), and the groups are merged through LDS.  With
+// nsplit > 1 every workgroup leaves (max, sum, output) of its range in the workspace and a second, small kernel
+// merges the ranges of a head (a merge by the workgroup that finishes last would need device-scope fences, which
+// write back and invalidate whole L2 caches on this multi-die GPU: measured 110 us per launch).
 template <int DT, int D>
 __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionParams p) {
     using E = Elem<DT>;
-    constexpr int LPP = D / 8, PPW = 64 / LPP, NG = 16 * PPW;
+    constexpr int LPP = D / 8, PPW = 64 / LPP, NG = 16 * PPW, UN = 4;
     extern __shared__ __align__(16) unsigned char smem[];
-    float* pm = (float*)smem;               // [NG]
-    float* pl = pm + NG;                    // [NG]
-    float* po = pl + NG;                    // [NG][D]
+    float* pm = (float*)smem;               // [NG] maxima
+    float* pw = pm + NG;                    // [NG] merge weights
+    float* pl = pw + NG;                    // [NG] sums
+    float* po = pl + NG;                    // [NG][D] outputs
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t sub = lane / LPP, dl = lane % LPP;
-    const uint32_t h = blockIdx.x, kvh = h / (p.n_head / p.n_kv);
+    const uint32_t nsplit = p.nsplit, h = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
+    const uint32_t kvh = h / (p.n_head / p.n_kv);
+    const uint16_t* kc = (const uint16_t*)p.k_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
+    const uint16_t* vc = (const uint16_t*)p.v_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
     long long pos64 = *p.pos;
+    uint32_t qr[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qr[e] = *(const uint32_t*)((const uint16_t*)p.q + (size_t)h * D + 8 * dl + 2 * e);
     if (pos64 < 0) pos64 = 0;
     const uint32_t len = (uint32_t)((pos64 + 1 < (long long)p.max_seq) ? pos64 + 1 : (long long)p.max_seq);
+    // this workgroup's positions: [lo, hi), ranges of a multiple of 16 PPW positions
+    const uint32_t chunk = ((len + nsplit - 1u) / nsplit + 16u * PPW - 1u) / (16u * PPW) * (16u * PPW);
+    const uint32_t lo = split * chunk < len ? split * chunk : len;
+    const uint32_t hi = (lo + chunk) < len ? (lo + chunk) : len;
     float q[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) q[e] = E::load(p.q, (size_t)h * D + 8 * dl + e) * p.scale;
+    for (int e = 0; e < 4; ++e) {
+        q[2 * e] = E::from_raw(qr[e] & 0xFFFFu) * p.scale;
+        q[2 * e + 1] = E::from_raw(qr[e] >> 16) * p.scale;
+    }
     float m = -__builtin_inff(), l = 0.f, o[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = 0.f;
-    const uint16_t* kc = (const uint16_t*)p.k_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
-    const uint16_t* vc = (const uint16_t*)p.v_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
-    for (uint32_t p0 = wave * PPW; p0 < len; p0 += 16 * PPW) {
-        const uint32_t pp = p0 + sub;
-        const bool valid = pp < len;
-        const uint32_t ppc = valid ? pp : len - 1u;
-        const u32x4 kr = *(const u32x4*)(kc + (size_t)ppc * D);
-        const u32x4 vr = *(const u32x4*)(vc + (size_t)ppc * D);
-        float s = 0.f;
+    for (uint32_t p0 = lo + wave * PPW; p0 < hi; p0 += UN * 16 * PPW) {
+        u32x4 kr[UN], vr[UN];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            s += q[2 * e] * E::from_raw(kr[e] & 0xFFFFu);
-            s += q[2 * e + 1] * E::from_raw(kr[e] >> 16);
+        for (int u = 0; u < UN; ++u) {
+            const uint32_t pp = p0 + (uint32_t)u * 16 * PPW + sub;
+            const uint32_t ppc = pp < hi ? pp : hi - 1u;
+            kr[u] = *(const u32x4*)(kc + (size_t)ppc * D);
+            vr[u] = *(const u32x4*)(vc + (size_t)ppc * D);
         }
-        s = group_sum<LPP>(s);
-        if (valid) {
-            const float mn = s > m ? s : m;
-            const float corr = __expf(m - mn), pr = __expf(s - mn);        // m = -inf: corr = 0
-            l = l * corr + pr;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const bool valid = p0 + (uint32_t)u * 16 * PPW + sub < hi;
+            float s = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                o[2 * e] = o[2 * e] * corr + pr * E::from_raw(vr[e] & 0xFFFFu);
-                o[2 * e + 1] = o[2 * e + 1] * corr + pr * E::from_raw(vr[e] >> 16);
+                s += q[2 * e] * E::from_raw(kr[u][e] & 0xFFFFu);
+                s += q[2 * e + 1] * E::from_raw(kr[u][e] >> 16);
             }
-            m = mn;
+            s = group_sum<LPP>(s);
+            if (valid) {
+                const float mn = s > m ? s : m;
+                const float corr = __expf(m - mn), pr = __expf(s - mn);        // m = -inf: corr = 0
+                l = l * corr + pr;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o[2 * e] = o[2 * e] * corr + pr * E::from_raw(vr[u][e] & 0xFFFFu);
+                    o[2 * e + 1] = o[2 * e + 1] * corr + pr * E::from_raw(vr[u][e] >> 16);
+                }
+                m = mn;
+            }
         }
     }
     const uint32_t g = wave * PPW + sub;
@@ -105,17 +128,65 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
 #pragma unroll
     for (int e = 0; e < 8; ++e) po[(size_t)g * D + 8 * dl + e] = o[e];
     __syncthreads();
-    if (tid < (uint32_t)D) {
-        float M = -__builtin_inff();
+    // merge of the NG groups: thread i < NG turns group i's maximum into its weight exp(m_i - M) (M = overall
+    // maximum, found by every such thread from the NG maxima), then thread d < D sums column d
+    float M = -__builtin_inff();
+    if (tid < (uint32_t)NG || tid < (uint32_t)D) {
         for (int i = 0; i < NG; ++i) M = pm[i] > M ? pm[i] : M;
-        float L = 0.f, O = 0.f;
+    }
+    if (tid < (uint32_t)NG) {
+        const float mi = pm[tid];
+        pw[tid] = (mi == -__builtin_inff()) ? 0.f : __expf(mi - M);
+    }
+    __syncthreads();
+    float L = 0.f, O = 0.f;
+    if (tid < (uint32_t)D) {
+#pragma unroll 8
         for (int i = 0; i < NG; ++i) {
-            const float w = (pm[i] == -__builtin_inff()) ? 0.f : __expf(pm[i] - M);
+            const float w = pw[i];
             L += pl[i] * w;
             O += po[(size_t)i * D + tid] * w;
         }
-        E::store(p.out, (size_t)h * D + tid, O / L);
     }
+    if (nsplit == 1u) {
+        if (tid < (uint32_t)D) E::store(p.out, (size_t)h * D + tid, O / L);
+        return;
+    }
+    // partial result of this range: [D] outputs, then the maximum and the sum; a second kernel merges them
+    float* ws = p.workspace + ((size_t)h * nsplit + split) * (D + 2);
+    if (tid < (uint32_t)D) {
+        ws[tid] = O;
+        if (tid == 0) { ws[D] = M; ws[D + 1] = L; }
+    }
+}
+
+// Second step with nsplit > 1: one workgroup of D threads per head combines the ranges' partial results.
+template <int DT, int D>
+__global__ __launch_bounds__(D) void decode_attention_merge_kernel(const AttentionParams p) {
+    using E = Elem<DT>;
+    const uint32_t tid = threadIdx.x, h = blockIdx.x, nsplit = p.nsplit;
+    const float* wh = p.workspace + (size_t)h * nsplit * (D + 2);
+    float ms[8], ls[8], os[8];
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) {
+        const uint32_t c = (uint32_t)sp < nsplit ? (uint32_t)sp : 0u;          // all loads in flight together
+        ms[sp] = wh[(size_t)c * (D + 2) + D];
+        ls[sp] = wh[(size_t)c * (D + 2) + D + 1];
+        os[sp] = wh[(size_t)c * (D + 2) + tid];
+    }
+    float Mg = -__builtin_inff();
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) if ((uint32_t)sp < nsplit && ms[sp] > Mg) Mg = ms[sp];
+    float Lg = 0.f, Og = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) {
+        if ((uint32_t)sp < nsplit) {
+            const float w = (ms[sp] == -__builtin_inff()) ? 0.f : __expf(ms[sp] - Mg);
+            Lg += ls[sp] * w;
+            Og += os[sp] * w;
+        }
+    }
+    E::store(p.out, (size_t)h * D + tid, Og / Lg);
 }
 
 template <int DT>
@@ -226,17 +297,28 @@ hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s) {
 
 size_t decode_attention_lds_bytes(uint32_t head_dim) {
     const size_t ng = 16 * (64 / (head_dim / 8));
-    return ng * (head_dim + 2) * sizeof(float);
+    return ng * (head_dim + 3) * sizeof(float);
 }
 
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s) {
-    const dim3 grid(p.n_head), block(1024);
+    const dim3 grid(p.n_head * p.nsplit), block(1024), mgrid(p.n_head);
     const size_t lds = decode_attention_lds_bytes(p.head_dim);
-    if (dt == kFP16 && p.head_dim == 128) hipLaunchKernelGGL((decode_attention_kernel<kFP16, 128>), grid, block, lds, s, p);
-    else if (dt == kFP16 && p.head_dim == 64) hipLaunchKernelGGL((decode_attention_kernel<kFP16, 64>), grid, block, lds, s, p);
-    else if (dt == kBF16 && p.head_dim == 128) hipLaunchKernelGGL((decode_attention_kernel<kBF16, 128>), grid, block, lds, s, p);
-    else if (dt == kBF16 && p.head_dim == 64) hipLaunchKernelGGL((decode_attention_kernel<kBF16, 64>), grid, block, lds, s, p);
-    else return hipErrorInvalidValue;
+    const bool merge = p.nsplit > 1;
+    if (dt == kFP16 && p.head_dim == 128) {
+        hipLaunchKernelGGL((decode_attention_kernel<kFP16, 128>), grid, block, lds, s, p);
+        if (merge) hipLaunchKernelGGL((decode_attention_merge_kernel<kFP16, 128>), mgrid, dim3(128), 0, s, p);
+    } else if (dt == kFP16 && p.head_dim == 64) {
+        hipLaunchKernelGGL((decode_attention_kernel<kFP16, 64>), grid, block, lds, s, p);
+        if (merge) hipLaunchKernelGGL((decode_attention_merge_kernel<kFP16, 64>), mgrid, dim3(64), 0, s, p);
+    } else if (dt == kBF16 && p.head_dim == 128) {
+        hipLaunchKernelGGL((decode_attention_kernel<kBF16, 128>), grid, block, lds, s, p);
+        if (merge) hipLaunchKernelGGL((decode_attention_merge_kernel<kBF16, 128>), mgrid, dim3(128), 0, s, p);
+    } else if (dt == kBF16 && p.head_dim == 64) {
+        hipLaunchKernelGGL((decode_attention_kernel<kBF16, 64>), grid, block, lds, s, p);
+        if (merge) hipLaunchKernelGGL((decode_attention_merge_kernel<kBF16, 64>), mgrid, dim3(64), 0, s, p);
+    } else {
+        return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

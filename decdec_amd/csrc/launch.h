@@ -59,6 +59,8 @@ struct AttentionParams {
     void* out;                       // [n_head * head_dim]
     uint32_t n_head, n_kv, head_dim, max_seq;
     float scale;
+    uint32_t nsplit;                 // workgroups per head (1: no workspace needed)
+    float* workspace;                // [n_head][nsplit][head_dim + 2] floats
 };
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);

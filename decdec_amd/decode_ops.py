@@ -28,15 +28,25 @@ def rope_cache_update(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: tor
                                                     _ptr(k_cache), _ptr(v_cache), _dt(qkv), n_head, n_kv_head, D, max_seq, _stream()))
 
 
+def attention_workspace(n_head: int, head_dim: int, device="cuda") -> torch.Tensor:
+    """Workspace that lets `decode_attention` share the positions of a head among 8 workgroups."""
+    n = _lib.load().decdec_decode_attention_workspace_bytes(n_head, head_dim, 8)
+    return torch.zeros(n // 4, dtype=torch.float32, device=device)
+
+
 def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor,
-                     out: torch.Tensor, n_head: int, n_kv_head: int) -> None:
+                     out: torch.Tensor, n_head: int, n_kv_head: int, workspace: torch.Tensor | None = None) -> None:
     _half_cuda(q, k_cache, v_cache, out)
     _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64 on the device")
     D, max_seq = k_cache.shape[-1], k_cache.shape[-2]
     _check(q.numel() == n_head * D and out.numel() == n_head * D, "q / out size mismatch")
     _check(k_cache.numel() == n_kv_head * max_seq * D and v_cache.shape == k_cache.shape, "cache shape mismatch")
+    if workspace is not None:
+        _check(workspace.is_cuda and workspace.is_contiguous() and workspace.dtype == torch.float32, "workspace must be a contiguous float32 CUDA tensor")
     _lib.check(_lib.load().decdec_decode_attention(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(out), _dt(q),
-                                                   n_head, n_kv_head, D, max_seq, _stream()))
+                                                   n_head, n_kv_head, D, max_seq,
+                                                   _ptr(workspace) if workspace is not None else None,
+                                                   workspace.numel() * 4 if workspace is not None else 0, _stream()))
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:

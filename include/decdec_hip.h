@@ -154,7 +154,10 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     writes the rotated queries to q_out and the rotated keys and the values into row `pos` of the caches
  *     ([n_kv_head][max_seq][head_dim]).  A position outside [0, max_seq) writes nothing.
  *   decdec_decode_attention: out[h] = softmax(q[h] . K[kv(h)][0..pos] / sqrt(head_dim)) V[kv(h)][0..pos],
- *     head_dim 64 or 128, grouped-query heads (kv(h) = h / (n_head / n_kv_head)).
+ *     head_dim 64 or 128, grouped-query heads (kv(h) = h / (n_head / n_kv_head)).  With a workspace of
+ *     decdec_decode_attention_workspace_bytes(n_head, head_dim, 8) bytes (caller-owned device memory, contents
+ *     irrelevant; one workspace serves any number of calls that do not overlap in time) the positions of a head
+ *     are shared by 8 workgroups and a second small kernel merges them; workspace NULL = one workgroup per head.
  *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n.
  *   decdec_add_rmsnorm: per row of `dim` elements (a multiple of 4, <= 16384; 8-byte aligned tensors), h = x + y rounded to the storage type and written to
  *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight. */
@@ -162,9 +165,11 @@ int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void*
                              const int64_t* pos_device, void* q_out, void* k_cache, void* v_cache,
                              int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
                              uint32_t max_seq, void* stream);
+uint64_t decdec_decode_attention_workspace_bytes(uint32_t n_head, uint32_t head_dim, uint32_t nsplit);
 int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache,
                             const int64_t* pos_device, void* out, int dtype, uint32_t n_head,
-                            uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream);
+                            uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq,
+                            void* workspace, uint64_t workspace_bytes, void* stream);
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
 int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
                        int dtype, uint32_t rows, uint32_t dim, float eps, void* stream);

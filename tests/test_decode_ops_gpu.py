@@ -52,15 +52,19 @@ def test_decode_attention(H, Hkv, hd, S, dt):
     g = torch.Generator(device="cuda").manual_seed(1)
     kc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
     vc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    ws = D.attention_workspace(H, hd)
     for pos in sorted({0, 1, 15, 16, 63, 64, S // 2 + 3, S - 1}):
         q = (torch.randn(H * hd, generator=g, device="cuda") * 1.5).to(dt)
         out = torch.empty(H * hd, dtype=dt, device="cuda")
         D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out, H, Hkv)
+        out_s = torch.empty(H * hd, dtype=dt, device="cuda")        # positions shared by 8 workgroups per head
+        D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out_s, H, Hkv, ws)
         k = kc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)       # [H, L, hd]
         v = vc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)
         att = torch.softmax(torch.einsum("hd,hld->hl", q.float().view(H, hd), k) / math.sqrt(hd), dim=-1)
         want = torch.einsum("hl,hld->hd", att, v)
         assert _close(out.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos,)
+        assert _close(out_s.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos, "split")
     # a position beyond the cache attends the whole cache and reads nothing outside it
     D.decode_attention(q, kc, vc, torch.tensor([S + 100], device="cuda"), out, H, Hkv)
     torch.cuda.synchronize()
