@@ -56,6 +56,8 @@ struct Options {
     int anyprec_rg = 0;
     int dec_block_waves = 16;   // waves of a standalone DEC workgroup: 4, 8 or 16
     int fused_two_per_cu = -1;  // fused launches: 1 / 0 = always / never two workgroups per compute unit, -1 = by estimate
+    int fused_small = -1;       // fused 3-bit any-precision launches with both roles in the GEMV's own smaller workgroups:
+                                // -1 = when those have 5..8 waves (measured faster there), 1 = whenever they have <= 8, 0 = never
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
@@ -79,6 +81,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "anyprec_rg")) return &g_opt.anyprec_rg;
     if (!strcmp(name, "anyprec_tile")) return &g_opt.anyprec_tile;
     if (!strcmp(name, "fused_two_per_cu")) return &g_opt.fused_two_per_cu;
+    if (!strcmp(name, "fused_small")) return &g_opt.fused_small;
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     return nullptr;
 }
@@ -204,7 +207,7 @@ struct Config {
     const void* thresholds_host;    // borrowed
     uint32_t K, N, M, k_chunk, max_smem;
     decdec_config_info info;
-    DecPlan plan;
+    DecPlan plans[3];               // for DEC workgroups of 4, 8 and 16 waves
     hipEvent_t e1, e2;
 };
 
@@ -222,10 +225,10 @@ Config* get_config(uint64_t h) {
 
 constexpr size_t kLdsBudget = 60 * 1024;
 
-// Split the DEC work of one layer over at most `budget` workgroups: cg chunk groups x sg segment
-// groups, minimising the longest per-workgroup path; ties prefer fewer chunk groups (= fewer atomic
+// Split the DEC work of one layer over at most `budget` workgroups of `nw` waves: cg chunk groups x sg
+// segment groups, minimising the longest per-workgroup path; ties prefer fewer chunk groups (= fewer atomic
 // adds per output).  The row list of a workgroup must fit in LDS.
-int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, DecPlan* pl) {
+int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t nw, DecPlan* pl) {
     const uint32_t num_chunks = cdiv(K, 1024);
     const uint32_t nseg = cdiv(M, 64);
     budget = std::max(1u, budget);
@@ -237,12 +240,12 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, DecPlan*
         for (uint32_t sg = 1; sg <= sg_max; ++sg) {
             const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
             const uint32_t slots = (cpb * std::max(k_chunk, 1u) + 1u) & ~1u;   // even: keeps the LDS arrays behind the row list 16-byte aligned
-            const size_t lds = dec_lds_bytes(slots);
+            const size_t lds = dec_lds_bytes(slots, nw);
             if (lds > kLdsBudget) continue;
             // per-workgroup critical path: sequential chunk selections, then batches of eight rows per
-            // wave for each group of up to 16 segments; going over the workgroup budget is a last resort
-            const uint32_t sb = std::min(spb, 16u), rl = 16u / sb;
-            const uint64_t batches = (uint64_t)cdiv(spb, 16) * cdiv(slots, rl * 8);
+            // wave for each group of up to nw segments; going over the workgroup budget is a last resort
+            const uint32_t sb = std::min(spb, nw), rl = nw / sb;
+            const uint64_t batches = (uint64_t)cdiv(spb, nw) * cdiv(slots, rl * 8);
             const uint64_t cost = batches * 1000 + (uint64_t)cpb * 600 + (uint64_t)cg * 10 +
                                   (cg * sg > budget ? 500000ull : 0);
             if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
@@ -266,21 +269,29 @@ int setup_config(Config* c, uint32_t k_chunk) {
     // reference dec_config.cu:180-181
     DD_CHECK(ctx->buffer_numel >= k, "DECContext buffer size is too small for the given k_chunk.");
     DD_CHECK(k_chunk <= 1024, "k_chunk must not exceed the chunk size (1024), got %u", k_chunk);
-    if (plan_dec(c->K, c->M, k_chunk, std::max(1u, ctx->num_tb), &c->plan))
-        return fail(kUnsupported, "DEC launch plan does not fit in LDS (k_chunk=%u, K=%u)", k_chunk, c->K);
-    c->info.hip_dec_blocks = (int)(c->plan.cg * c->plan.sg);
-    c->info.hip_chunk_groups = (int)c->plan.cg;
-    c->info.hip_segment_groups = (int)c->plan.sg;
-    c->info.hip_vec_words = (int)c->plan.vec;
-    c->info.hip_lds_bytes = (int)c->plan.lds;
-    c->info.hip_slots_per_block = (int)c->plan.slots;
-    c->info.hip_lds_reduce = (int)c->plan.lds_reduce;
+    // num_tb counts 1024-thread workgroups; smaller workgroups get the same number of waves in total
+    for (uint32_t i = 0; i < 3; ++i) {
+        const uint32_t nw = 4u << i;
+        if (plan_dec(c->K, c->M, k_chunk, std::max(1u, ctx->num_tb) * (16u / nw), nw, &c->plans[i]))
+            return fail(kUnsupported, "DEC launch plan does not fit in LDS (k_chunk=%u, K=%u)", k_chunk, c->K);
+    }
+    const DecPlan& plan = c->plans[2];
+    c->info.hip_dec_blocks = (int)(plan.cg * plan.sg);
+    c->info.hip_chunk_groups = (int)plan.cg;
+    c->info.hip_segment_groups = (int)plan.sg;
+    c->info.hip_vec_words = (int)plan.vec;
+    c->info.hip_lds_bytes = (int)plan.lds;
+    c->info.hip_slots_per_block = (int)plan.slots;
+    c->info.hip_lds_reduce = (int)plan.lds_reduce;
     c->info.hip_residual_on_host = c->residual_host != nullptr;
     return kOk;
 }
 
 // Fill the kernel parameters of one DEC call.  Returns 1 when there is nothing to do (k == 0).
-int fill_dec_params(const Config* c, const void* input, void* output, bool fused_select, DecParams* p) {
+const DecPlan& dec_plan(const Config* c, uint32_t nw) { return c->plans[nw <= 4 ? 0 : (nw <= 8 ? 1 : 2)]; }
+
+int fill_dec_params(const Config* c, const void* input, void* output, bool fused_select, DecParams* p,
+                    uint32_t nw = kDecWaves) {
     const uint64_t k = (uint64_t)c->k_chunk * c->K / 1024;       // reference decdec.cu:50
     if (k == 0) return 1;                                        // reference decdec.cu:52-54
     memset(p, 0, sizeof(*p));
@@ -297,8 +308,9 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
     }
     p->K = c->K; p->N = c->N; p->M = c->M;
     p->num_chunks = cdiv(c->K, 1024); p->k_chunk = c->k_chunk; p->k_total = (uint32_t)k;
-    p->cg = c->plan.cg; p->sg = c->plan.sg; p->nseg = c->plan.nseg;
-    p->segs_per_block = c->plan.segs_per_block; p->slots_per_block = c->plan.slots;
+    const DecPlan& plan = dec_plan(c, nw);
+    p->cg = plan.cg; p->sg = plan.sg; p->nseg = plan.nseg;
+    p->segs_per_block = plan.segs_per_block; p->slots_per_block = plan.slots;
     p->fused_select = fused_select ? 1u : 0u;
     if (g_opt.dec_trace && p->cg * p->sg <= (uint32_t)kTraceBlocks) {
         if (!g_trace_dev && hipMalloc(&g_trace_dev, sizeof(unsigned long long) * 8 * kTraceBlocks) != hipSuccess)
@@ -343,7 +355,6 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     p.sgroups = cdiv(s_total, 16);
     p.S = cdiv(s_total, p.sgroups);
     p.rg = fused_block ? std::max(1u, 16u / p.S) : std::max(1u, 4u / p.S);   // 256-thread workgroups measured best
-    if (!fused_block && g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
     // Rows per wave: every wave requests all its rows at once, so more rows per wave mean more bytes
     // in flight per resident wave (large matrices), fewer rows mean more waves to share the decode
     // work (small matrices, where one wave per SIMD would issue at a quarter of the VALU rate).
@@ -352,6 +363,7 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     if (row_slices >= 16384 && p.S * p.sgroups >= 4) rpw = 8u;     // long rows (K >= 8192): measured 9.0 against 10.1 us at 14336 -> 4096
     if (g_opt.anyprec_rpw == 2 || g_opt.anyprec_rpw == 4 || g_opt.anyprec_rpw == 8) rpw = (uint32_t)g_opt.anyprec_rpw;
     p.rpw = rpw;
+    if (g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
     p.x_aligned = ((uintptr_t)input % 16) == 0;
     pl->d.grid = cdiv(N, p.rg * p.rpw) * p.sgroups;
     pl->d.block = fused_block ? 1024u : 64u * p.S * p.rg;
@@ -459,7 +471,8 @@ static int two_stream(Config* c, const DecParams* dp, bool have_dec, int dtype, 
     hipStream_t sub = c->ctx->sub_stream;
     DD_HIP(hipEventRecord(c->e1, main_stream));
     if (have_dec) {
-        LaunchDims d{c->plan.cg * c->plan.sg, dec_block_threads(), c->plan.lds};
+        const DecPlan& plan = dec_plan(c, kDecWaves);
+        LaunchDims d{plan.cg * plan.sg, (uint32_t)kDecThreads, plan.lds};
         DD_HIP(launch_dec(dtype, *dp, d, main_stream));
     }
     DD_HIP(hipStreamWaitEvent(sub, c->e1, 0));
@@ -685,8 +698,10 @@ static int dec_common(uint64_t h, const void* input, void* output, int dtype, ui
     int rc = check_dec_call(c, dtype, K, N, input, output);
     if (rc != kOk) return rc;
     DecParams p;
-    if (fill_dec_params(c, input, output, fused_select, &p)) return kOk;
-    LaunchDims d{c->plan.cg * c->plan.sg, dec_block_threads(), c->plan.lds};
+    const uint32_t nw = dec_block_threads() / kWave;
+    if (fill_dec_params(c, input, output, fused_select, &p, nw)) return kOk;
+    const DecPlan& plan = dec_plan(c, nw);
+    LaunchDims d{plan.cg * plan.sg, nw * kWave, plan.lds};
     DD_HIP(launch_dec(dtype, p, d, (hipStream_t)stream));
     return kOk;
 }
@@ -743,12 +758,27 @@ int decdec_sqllm_gemv(const void* input, void* output, const void* mat, const vo
 // GEMV role is expected to outlast the DEC role by a margin.  Estimates in microseconds: DEC = its latency
 // floor (launch, activation load, selection, one host-link round trip, merge: about 8) plus the residual
 // bytes at the zero-copy rate of the link (56 GB/s); GEMV = 2 plus its weight bytes at 2.5 TB/s.
+double dec_estimate_us(const Config* c) {
+    const double k = (double)((uint64_t)c->k_chunk * c->K / 1024u);        // selected rows per call
+    return 8.0 + k * (double)c->N * 0.5 / 56e3;
+}
+double gemv_estimate_us(double gemv_bytes) { return 2.0 + gemv_bytes / 2.5e6; }
+
 bool fused_two_per_cu(const Config* c, double gemv_bytes) {
     if (g_opt.fused_two_per_cu >= 0) return g_opt.fused_two_per_cu != 0;
-    const double k = (double)((uint64_t)c->k_chunk * c->K / 1024u);        // selected rows per call
-    const double dec_us = 8.0 + k * (double)c->N * 0.5 / 56e3;
-    const double gemv_us = 2.0 + gemv_bytes / 2.5e6;
-    return gemv_us > 1.25 * dec_us;
+    return gemv_estimate_us(gemv_bytes) > 1.25 * dec_estimate_us(c);
+}
+
+// Whether a fused 3-bit any-precision launch runs both roles in workgroups of `nw` waves (the GEMV's standalone
+// size).  Measured at 14336 -> 4096 (8 waves): 12.0 / 12.6 / 14.6 us against 13.3 / 16.4 / 15.9 us for the
+// 1024-thread form at k_chunk 1 / 4 / 8, but 16.7 against 15.9 us at k_chunk 12 and 26.5 against 24.0 us at 32: a
+// DEC workgroup's host-memory reads hold up the GEMV waves of its compute unit, and the small form spreads the DEC
+// workgroups over four times as many units, so it only pays while the GEMV is the longer role.  With 4-wave
+// workgroups (K <= 8192) the 1024-thread form was as fast or faster at every k_chunk.
+bool fused_small(const Config* c, double gemv_bytes, uint32_t nw) {
+    if (nw >= 16u || g_opt.fused_small == 0) return false;
+    if (g_opt.fused_small > 0) return true;
+    return nw == 8u && dec_estimate_us(c) < 1.2 * gemv_estimate_us(gemv_bytes);
 }
 
 int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
@@ -762,14 +792,30 @@ int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* 
     const bool fuse = g_opt.fusion && have_dec;
     AnyprecPlan pl;
     const bool two = fuse && bits == 3 && fused_two_per_cu(c, (double)bits * N * K / 8.0);
+    hipStream_t s = (hipStream_t)stream;
+    if (fuse && bits == 3 && g_opt.fused_small != 0) {
+        // Both roles in workgroups of the GEMV's own size (4 or 8 waves): the GEMV keeps its standalone
+        // schedule and a DEC workgroup holds an eighth or a quarter of a compute unit instead of a half.
+        rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, false, &pl);
+        if (rc != kOk) return rc;
+        const uint32_t nw = pl.d.block <= 256u ? 4u : (pl.d.block <= 512u ? 8u : 16u);
+        if (pl.p.tile_cs == 0u && fused_small(c, (double)bits * N * K / 8.0, nw)) {
+            (void)fill_dec_params(c, input, output, true, &dp, nw);
+            const DecPlan& plan = dec_plan(c, nw);
+            LaunchDims d = pl.d;
+            d.block = nw * kWave;
+            d.lds = std::max(d.lds, plan.lds);
+            DD_HIP(launch_dec_anyprec_small(dtype, nw, dp, plan.cg * plan.sg, pl.p, d, s));
+            return kOk;
+        }
+    }
     rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, fuse, &pl);
     if (rc != kOk) return rc;
-    hipStream_t s = (hipStream_t)stream;
     if (fuse) {
         LaunchDims d = pl.d;
-        d.lds = std::max(d.lds, c->plan.lds);
+        d.lds = std::max(d.lds, c->plans[2].lds);
         d.two_per_cu = two;
-        DD_HIP(launch_dec_anyprec(dtype, bits, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        DD_HIP(launch_dec_anyprec(dtype, bits, dp, c->plans[2].cg * c->plans[2].sg, pl.p, d, s));
         return kOk;
     }
     if (!have_dec && g_opt.fusion) { DD_HIP(launch_anyprec(dtype, bits, pl.p, pl.d, s)); return kOk; }
@@ -792,9 +838,9 @@ int decdec_dec_lutgemm(uint64_t h, const void* input, void* output, const void* 
     hipStream_t s = (hipStream_t)stream;
     if (fuse) {
         LaunchDims d = pl.d;
-        d.lds = std::max(d.lds, c->plan.lds);
+        d.lds = std::max(d.lds, c->plans[2].lds);
         d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
-        DD_HIP(launch_dec_lutgemm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        DD_HIP(launch_dec_lutgemm(dtype, dp, c->plans[2].cg * c->plans[2].sg, pl.p, d, s));
         return kOk;
     }
     if (!have_dec && g_opt.fusion) { DD_HIP(launch_lutgemm(dtype, pl.p, pl.d, s)); return kOk; }
@@ -815,9 +861,9 @@ int decdec_dec_sqllm(uint64_t h, const void* input, void* output, const void* ma
     hipStream_t s = (hipStream_t)stream;
     if (fuse) {
         LaunchDims d = pl.d;
-        d.lds = std::max(d.lds, c->plan.lds);
+        d.lds = std::max(d.lds, c->plans[2].lds);
         d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
-        DD_HIP(launch_dec_sqllm(dtype, dp, c->plan.cg * c->plan.sg, pl.p, d, s));
+        DD_HIP(launch_dec_sqllm(dtype, dp, c->plans[2].cg * c->plans[2].sg, pl.p, d, s));
         return kOk;
     }
     if (!have_dec && g_opt.fusion) { DD_HIP(launch_sqllm(dtype, pl.p, pl.d, s)); return kOk; }

@@ -54,8 +54,8 @@ constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per
 
 __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves = kDecWaves) {
     // row list (index + activation) + selection counters/prefix + the buffer shared by the cross-wave
-    // reduction ([nwaves][8][64] floats) and the partial ranks of the selection ([16][kMaxCand])
-    const size_t red = (size_t)nwaves * 8 * kWave * 4, ranks = (size_t)16 * kMaxCand * 4;
+    // reduction ([nwaves][8][64] floats) and the partial ranks of the selection ([16][kMaxCand] bytes)
+    const size_t red = (size_t)nwaves * 8 * kWave * 4, ranks = (size_t)16 * kMaxCand;
     return (size_t)slots * 8 + 2 * 512 * 4 + (red > ranks ? red : ranks);
 }
 
@@ -196,7 +196,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
     uint32_t* key = cnt + 32;                              // [kMaxCand]
     float* cx = (float*)(cnt + 32 + kMaxCand);             // [kMaxCand] (runs into `pre`, unused here)
     uint32_t* hdr = cnt + 32 + 2 * kMaxCand;               // fast flag, candidate count
-    uint32_t* pc = (uint32_t*)red;                         // [16][kMaxCand] partial ranks
+    uint8_t* pc = (uint8_t*)red;                           // [16][kMaxCand] partial ranks (each at most 16)
     const bool scanner = p.monotone && wave < (uint32_t)kSelWaves;   // uniform per wave
 
     // ---- four waves scan the chunk: lane l of wave w owns channels 4 (64 w + l) .. + 3
@@ -338,7 +338,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
                 const u32x4 k4 = kp[v];
                 r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
             }
-            pc[iq * kMaxCand + j] = r;
+            pc[iq * kMaxCand + j] = (uint8_t)r;
         }
     }
     __syncthreads();

@@ -18,6 +18,16 @@ __global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_anyprec_kernel(co
     else anyprec_role<DT, BITS>(gp, blockIdx.x - dec_blocks, smem);
 }
 
+// The same two roles in workgroups of NW (4 or 8) waves, eight waves per SIMD: the GEMV role runs in workgroups of
+// its standalone size, and a DEC workgroup holds an eighth or a quarter of a compute unit.
+template <int DT, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(8, 8)))
+void dec_anyprec3_small_kernel(const DecParams dp, const uint32_t dec_blocks, const AnyprecParams gp) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if (blockIdx.x < dec_blocks) dec_role<DT, NW>(dp, blockIdx.x, smem);
+    else anyprec_role<DT, 3>(gp, blockIdx.x - dec_blocks, smem);
+}
+
 // W[n][c] = lut[n][idx(n, c)]: one thread per (row, word); the 32 weights of a word go to four groups
 // of eight consecutive channels (reference dequant_kbit_store, decdec_extension/anyprec.cu:261-331).
 template <int DT, int BITS>
@@ -90,6 +100,20 @@ hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t de
         DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, B, false>), grid, block, d.lds, s, dp, dec_blocks, gp));
     } else {
         return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_anyprec_small(int dt, uint32_t nw, const DecParams& dp, uint32_t dec_blocks,
+                                    const AnyprecParams& gp, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(dec_blocks + d.grid), block(d.block);
+    if (d.block != nw * 64u || (nw != 4u && nw != 8u) || (dt != kFP16 && dt != kBF16)) return hipErrorInvalidValue;
+    if (dt == kFP16) {
+        if (nw == 4u) hipLaunchKernelGGL((dec_anyprec3_small_kernel<kFP16, 4>), grid, block, d.lds, s, dp, dec_blocks, gp);
+        else hipLaunchKernelGGL((dec_anyprec3_small_kernel<kFP16, 8>), grid, block, d.lds, s, dp, dec_blocks, gp);
+    } else {
+        if (nw == 4u) hipLaunchKernelGGL((dec_anyprec3_small_kernel<kBF16, 4>), grid, block, d.lds, s, dp, dec_blocks, gp);
+        else hipLaunchKernelGGL((dec_anyprec3_small_kernel<kBF16, 8>), grid, block, d.lds, s, dp, dec_blocks, gp);
     }
     return hipGetLastError();
 }

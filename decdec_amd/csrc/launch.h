@@ -35,6 +35,9 @@ hipError_t launch_burner(uint32_t blocks, long long iters, hipStream_t s);
 // d.grid counts the GEMV workgroups only; d.block is 1024.
 hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t dec_blocks,
                               const AnyprecParams& gp, const LaunchDims& d, hipStream_t s);
+// 3-bit, both roles in workgroups of `nw` (4 or 8) waves = d.block / 64; dp carries the DEC plan for that size.
+hipError_t launch_dec_anyprec_small(int dt, uint32_t nw, const DecParams& dp, uint32_t dec_blocks,
+                                    const AnyprecParams& gp, const LaunchDims& d, hipStream_t s);
 hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
                               const LutgemmParams& gp, const LaunchDims& d, hipStream_t s);
 hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,

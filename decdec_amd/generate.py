@@ -20,7 +20,7 @@ import time
 
 import torch
 
-from . import artifacts
+from . import _lib, artifacts
 from .linear import APLinear, LUTGEMMLinear, SQLLMLinear
 from .model import DEC_MODULE_KEYS, Transformer
 
@@ -198,7 +198,12 @@ def main(argv=None):
     ap.add_argument("--max-seq-length", type=int, default=2048)
     ap.add_argument("--n-layer", type=int, default=None, help="fewer layers than the named model (smoke runs)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="library option (decdec_set_option), e.g. fusion=0; may be repeated")
     args = ap.parse_args(argv)
+    for kv in args.option:
+        name, _, value = kv.partition("=")
+        _lib.set_option(name, int(value))
     if len(args.k_chunk) == 1:
         k_sets = [args.k_chunk * 4]
     else:

@@ -57,7 +57,10 @@ int decdec_version(void);
  * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "anyprec_tile" (3-bit LDS-transposed tile decoder, waves per tile 2/4/8, 0 = off [default]), "lutgemm_ktiles",
  * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "fused_two_per_cu" (fused launches: 1 / 0 = always /
  * never the kernel instance that lets two workgroups share a compute unit, -1 = chosen per launch [default]),
- * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]), "dec_trace" (see
+ * "fused_small" (fused 3-bit any-precision launches with both roles in the GEMV's own 4- or 8-wave workgroups:
+ * -1 = when those have 5 to 8 waves [default], 1 = whenever they have at most 8, 0 = never), "anyprec_rg" (row
+ * groups per any-precision workgroup, 0 = automatic),
+ * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
 int decdec_get_option(const char* name, int* value);

@@ -276,6 +276,36 @@ def test_fused_launch_with_two_workgroups_per_cu(kind, K, N, k_chunk, c_oracle):
     ext.destroy_dec_config(cfg)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K,N,k_chunk,n_tb", [(4096, 4096, 4, 16), (14336, 1032, 2, 8), (11008, 4096, 40, 32),
+                                               (1536, 2056, 8, 4), (8192, 1024, 100, 16), (5120, 7680, 1, 32)])
+def test_fused_anyprec_in_small_workgroups(dtype, K, N, k_chunk, n_tb, c_oracle):
+    """3-bit any-precision + DEC in one launch of 4- or 8-wave workgroups (the GEMV's standalone size, the DEC
+    role with the launch plan for that size), forced on for every shape that allows it: selection bit-exact,
+    output against the oracle."""
+    from decdec_amd import _lib
+    L = make_dec_layer(K, N, seed=K + N + k_chunk, dtype=dtype)
+    ctx, rows, acts = _ctx(n_tb, K, dtype)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+    x = L["x"].cuda()
+    out = torch.zeros(1, 1, N, dtype=dtype, device="cuda")
+    _lib.set_option("fused_small", 1)
+    try:
+        ext.dec_anyprec(cfg, x, out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_option("fused_small", -1)
+    want_rows, _, _ = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk,
+                                        "fp16" if dtype == torch.float16 else "bf16")
+    k = k_chunk * K // 1024
+    assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k])
+    base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+    want = base + c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows)
+    mre, mae = rel_err(np_of(out).reshape(-1), want)
+    assert mre <= (TOL if dtype == torch.float16 else TOL_BF16), (mre, mae)
+    ext.destroy_dec_config(cfg)
+
+
 def test_unfused_dec_uses_caller_indices(c_oracle):
     """evaluation/evaltools.py:327-343: exact top-k indices are written into the context's row
     buffer and unfused_dec fetches those rows."""
