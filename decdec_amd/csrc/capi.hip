@@ -539,6 +539,26 @@ int decdec_reference_geometry(uint32_t K, uint32_t N, uint32_t n_tb, uint32_t k_
     return kOk;
 }
 
+int decdec_dec_launch_plan(uint32_t K, uint32_t N, uint32_t n_tb, uint32_t k_chunk, uint32_t block_waves,
+                           decdec_config_info* out) {
+    DD_CHECK(out && n_tb >= 1 && K >= 1 && N >= 8 && N % 8 == 0, "invalid argument");
+    DD_CHECK(block_waves == 4 || block_waves == 8 || block_waves == 16, "block_waves must be 4, 8 or 16");
+    DD_CHECK(k_chunk <= 1024, "k_chunk must not exceed the chunk size (1024), got %u", k_chunk);
+    DecPlan pl;
+    if (plan_dec(K, N / 8, k_chunk, n_tb * (16u / block_waves), block_waves, &pl))
+        return fail(kUnsupported, "DEC launch plan does not fit in LDS (k_chunk=%u, K=%u)", k_chunk, K);
+    memset(out, 0, sizeof(*out));
+    out->num_chunks = (int)cdiv(K, 1024); out->chunk_size = 1024; out->k_chunk = (int)k_chunk;
+    out->hip_dec_blocks = (int)(pl.cg * pl.sg);
+    out->hip_chunk_groups = (int)pl.cg;
+    out->hip_segment_groups = (int)pl.sg;
+    out->hip_vec_words = (int)pl.vec;
+    out->hip_lds_bytes = (int)pl.lds;
+    out->hip_slots_per_block = (int)pl.slots;
+    out->hip_lds_reduce = (int)pl.lds_reduce;
+    return kOk;
+}
+
 // ---------------------------------------------------------------- context
 int decdec_create_dec_context(uint32_t num_tb, int dtype, uint64_t buffer_numel, void* rows, void* acts,
                               uint64_t* out) {

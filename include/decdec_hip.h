@@ -190,6 +190,13 @@ int decdec_bucket_floors(float threshold_a, float threshold_b, int dtype, float*
 int decdec_reference_geometry(uint32_t num_rows, uint32_t num_cols, uint32_t num_tb,
                               uint32_t k_chunk, int dtype, uint32_t max_shared_memory,
                               decdec_config_info* info_out);
+/* The library's own DEC launch plan for a shape (the hip_* fields of decdec_config_info, plus num_chunks,
+ * chunk_size, k_chunk) for DEC workgroups of `block_waves` (4, 8 or 16) waves: num_tb counts 1024-thread
+ * workgroups, smaller ones get the same number of waves in total.  Host-only; takes the place of the launch
+ * geometry of dec_config.cu:34-115, which it does not follow (one workgroup per chunk group x column-segment
+ * group, no grid barrier). */
+int decdec_dec_launch_plan(uint32_t num_rows, uint32_t num_cols, uint32_t num_tb, uint32_t k_chunk,
+                           uint32_t block_waves, decdec_config_info* info_out);
 
 #ifdef __cplusplus
 }

@@ -62,6 +62,31 @@ def test_library_reference_geometry_matches_oracle(K, N, n_tb, k_chunk):
         assert getattr(info, key) == want[key], key
 
 
+@pytest.mark.parametrize("waves", [4, 8, 16])
+def test_dec_launch_plan_covers_the_layer(waves):
+    """The DEC launch plan (host-only): every chunk and every 64-word column segment belongs to a workgroup, the row
+    list holds a chunk group's picks, LDS stays within the budget, the workgroup budget is kept wherever a plan
+    within it exists, and at decode shapes a workgroup fetches its segments in one batch."""
+    lib = _lib.load()
+    info = _lib.ConfigInfo()
+    for K in (1024, 1536, 4096, 5120, 8192, 11008, 14336, 17920, 28672):
+        for N in (8, 64, 1032, 4096, 7680, 14336, 28672, 35840):
+            for n_tb in (1, 8, 16, 32, 64):
+                for k_chunk in (1, 4, 32, 100, 1024):
+                    _lib.check(lib.decdec_dec_launch_plan(K, N, n_tb, k_chunk, waves, ctypes.byref(info)))
+                    chunks, nseg = -(-K // 1024), -(-(N // 8) // 64)
+                    cg, sg = info.hip_chunk_groups, info.hip_segment_groups
+                    assert 1 <= cg <= chunks and 1 <= sg <= nseg and info.hip_dec_blocks == cg * sg
+                    cpb, spb = -(-chunks // cg), -(-nseg // sg)
+                    assert info.hip_slots_per_block >= cpb * k_chunk and info.hip_slots_per_block % 2 == 0
+                    red = max(waves * 2048, 16 * 256)
+                    assert info.hip_lds_bytes == info.hip_slots_per_block * 8 + 4096 + red <= 60 * 1024
+                    budget = n_tb * (16 // waves)
+                    assert cg * sg <= budget or cg == 1 or chunks > budget, (K, N, n_tb, k_chunk, cg, sg)
+                    if k_chunk <= 32 and budget >= chunks * -(-nseg // waves):
+                        assert spb <= waves, (K, N, n_tb, k_chunk, cg, sg)
+
+
 def test_invalid_handles_and_arguments_fail_cleanly():
     lib = _lib.load()
     assert lib.decdec_destroy_dec_config(12345) != 0 and "invalid DECConfig handle" in _lib.last_error()
