@@ -54,13 +54,15 @@ SIGNATURES = {
     "decdec_decode_attention": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp, _u64, _vp],
     "decdec_silu_mul": [_vp, _vp, _i32, _u32, _vp],
     "decdec_add_rmsnorm": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp],
+    "decdec_greedy_pick": [_vp, _u32, _i32, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp],
     "decdec_debug_read_trace": [ctypes.POINTER(_u64), _i32],
     "decdec_bucket_floors": [_f32, _f32, _i32, ctypes.POINTER(_f32)],
     "decdec_reference_geometry": [_u32, _u32, _u32, _u32, _i32, _u32, ctypes.POINTER(ConfigInfo)],
     "decdec_dec_launch_plan": [_u32, _u32, _u32, _u32, _u32, ctypes.POINTER(ConfigInfo)],
 }
 OTHER_SYMBOLS = {"decdec_last_error": ([], ctypes.c_char_p), "decdec_version": ([], _i32),
-                 "decdec_decode_attention_workspace_bytes": ([_u32, _u32, _u32], _u64)}
+                 "decdec_decode_attention_workspace_bytes": ([_u32, _u32, _u32], _u64),
+                 "decdec_greedy_pick_workspace_bytes": ([], _u64)}
 
 
 def load():

@@ -971,6 +971,20 @@ int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void*
     return kOk;
 }
 
+uint64_t decdec_greedy_pick_workspace_bytes(void) { return (uint64_t)greedy_pick_workspace_bytes(); }
+
+int decdec_greedy_pick(const void* logits, uint32_t n, int dtype, void* workspace, float* logits_f32_out,
+                       int64_t* token, int64_t* seq, uint32_t seq_capacity, int64_t* count, int64_t* pos, void* stream) {
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
+    DD_CHECK(logits && workspace && token, "null pointer argument");
+    DD_CHECK(n >= 1, "there must be at least one logit");
+    DD_CHECK((seq == nullptr) == (count == nullptr), "seq and count go together");
+    DD_CHECK(((uintptr_t)workspace % 8) == 0, "workspace must be 8-byte aligned");
+    DD_HIP(launch_greedy_pick(dtype, logits, n, workspace, logits_f32_out, (long long*)token, (long long*)seq,
+                              seq_capacity, (long long*)count, (long long*)pos, (hipStream_t)stream));
+    return kOk;
+}
+
 int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out, int dtype,
                        uint32_t rows, uint32_t dim, float eps, void* stream) {
     DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");

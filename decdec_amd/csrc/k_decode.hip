@@ -286,6 +286,72 @@ hipError_t launch_add_rmsnorm(int dt, const void* x, const void* y, const void* 
     return hipErrorInvalidValue;
 }
 
+// ---- greedy pick: argmax of the logits and the bookkeeping of a decode step ---------------------------
+// Key of a logit: its value mapped to an unsigned integer that orders like the float (NaN with the sign bit
+// clear above +inf, as torch.argmax treats it), then the complement of the index, so that the largest key is
+// the largest logit and, among equal ones, the one with the smallest index.
+__device__ __forceinline__ unsigned long long pick_key(float v, uint32_t idx) {
+    const uint32_t b = __float_as_uint(v);
+    const uint32_t u = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return ((unsigned long long)u << 32) | (unsigned long long)(0xFFFFFFFFu - idx);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const unsigned long long o = __shfl_xor(k, off, 64);
+        k = o > k ? o : k;
+    }
+    return k;
+}
+
+constexpr int kPickBlocks = 128;      // partial results (and workgroups of the first kernel)
+
+template <int DT>
+__global__ __launch_bounds__(256) void greedy_partial_kernel(const void* __restrict__ logits, const uint32_t n,
+                                                            unsigned long long* __restrict__ partial,
+                                                            float* __restrict__ copy_out) {
+    using E = Elem<DT>;
+    __shared__ unsigned long long wk[4];
+    unsigned long long best = 0ull;                      // below every key of a real element
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += (uint32_t)kPickBlocks * 256u) {
+        const float v = E::load(logits, i);
+        if (copy_out != nullptr) copy_out[i] = v;
+        const unsigned long long k = pick_key(v, i);
+        best = k > best ? k : best;
+    }
+    best = wave_max_u64(best);
+    if ((threadIdx.x & 63u) == 0) wk[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long b = wk[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) b = wk[w] > b ? wk[w] : b;
+        partial[blockIdx.x] = b;
+    }
+}
+
+// One wave: reduces the partial keys, stores the token, appends it to the sequence, advances the position
+// and the count (all in device memory, so that a captured step needs no host value).
+__global__ __launch_bounds__(64) void greedy_final_kernel(const unsigned long long* __restrict__ partial,
+                                                         long long* __restrict__ token, long long* __restrict__ seq,
+                                                         const uint32_t seq_capacity, long long* __restrict__ count,
+                                                         long long* __restrict__ pos) {
+    unsigned long long best = 0ull;
+    for (uint32_t i = threadIdx.x; i < (uint32_t)kPickBlocks; i += 64u) best = partial[i] > best ? partial[i] : best;
+    best = wave_max_u64(best);
+    if (threadIdx.x == 0) {
+        const long long idx = (long long)(0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull));
+        token[0] = idx;
+        if (seq != nullptr && count != nullptr) {
+            const long long c = count[0];
+            if (c >= 0 && c < (long long)seq_capacity) seq[c] = idx;
+            count[0] = c + 1;
+        }
+        if (pos != nullptr) pos[0] += 1;
+    }
+}
+
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s) {
     const uint32_t threads = (p.n_head + p.n_kv) * (p.head_dim / 2) + p.n_kv * p.head_dim;
     const dim3 grid((threads + 255) / 256), block(256);
@@ -327,6 +393,19 @@ hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, h
     if (dt == kFP16) hipLaunchKernelGGL((silu_mul_kernel<kFP16>), grid, block, 0, s, gate_up, out, n);
     else if (dt == kBF16) hipLaunchKernelGGL((silu_mul_kernel<kBF16>), grid, block, 0, s, gate_up, out, n);
     else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+size_t greedy_pick_workspace_bytes() { return (size_t)kPickBlocks * sizeof(unsigned long long); }
+
+hipError_t launch_greedy_pick(int dt, const void* logits, uint32_t n, void* workspace, float* copy_out, long long* token,
+                              long long* seq, uint32_t seq_capacity, long long* count, long long* pos, hipStream_t s) {
+    unsigned long long* partial = (unsigned long long*)workspace;
+    if (dt == kFP16) hipLaunchKernelGGL((greedy_partial_kernel<kFP16>), dim3(kPickBlocks), dim3(256), 0, s, logits, n, partial, copy_out);
+    else if (dt == kBF16) hipLaunchKernelGGL((greedy_partial_kernel<kBF16>), dim3(kPickBlocks), dim3(256), 0, s, logits, n, partial, copy_out);
+    else if (dt == kFP32) hipLaunchKernelGGL((greedy_partial_kernel<kFP32>), dim3(kPickBlocks), dim3(256), 0, s, logits, n, partial, copy_out);
+    else return hipErrorInvalidValue;
+    hipLaunchKernelGGL(greedy_final_kernel, dim3(1), dim3(64), 0, s, partial, token, seq, seq_capacity, count, pos);
     return hipGetLastError();
 }
 

@@ -68,6 +68,9 @@ struct AttentionParams {
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);
 hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, hipStream_t s);
+size_t greedy_pick_workspace_bytes();
+hipError_t launch_greedy_pick(int dt, const void* logits, uint32_t n, void* workspace, float* copy_out, long long* token,
+                              long long* seq, uint32_t seq_capacity, long long* count, long long* pos, hipStream_t s);
 hipError_t launch_add_rmsnorm(int dt, const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
                               uint32_t rows, uint32_t dim, float eps, hipStream_t s);
 

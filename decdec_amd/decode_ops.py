@@ -67,3 +67,30 @@ def add_rmsnorm(x: torch.Tensor, y, weight: torch.Tensor, h_out, normed_out: tor
                                               _ptr(h_out) if h_out is not None else None, _ptr(normed_out), _dt(x),
                                               x.numel() // dim, dim, float(eps), _stream()))
 
+
+
+def greedy_pick_workspace(device="cuda") -> torch.Tensor:
+    """Workspace of `greedy_pick` (contents irrelevant; one serves any number of calls that do not overlap)."""
+    return torch.empty(int(_lib.load().decdec_greedy_pick_workspace_bytes()) // 8, dtype=torch.int64, device=device)
+
+
+def greedy_pick(logits: torch.Tensor, workspace: torch.Tensor, token: torch.Tensor, seq=None, count=None, pos=None,
+                logits_f32_out=None) -> None:
+    """token[0] = argmax(logits) (smallest index among equal logits); seq[count[0]] = it and count[0] += 1 when seq and
+    count are given; pos[0] += 1 when pos is given; logits_f32_out receives the logits as fp32 when given.  token, seq,
+    count and pos are int64 tensors on the device."""
+    _check(logits.is_cuda and logits.is_contiguous() and logits.dtype in (torch.float16, torch.bfloat16, torch.float32),
+           "logits must be a contiguous fp16 / bf16 / fp32 CUDA tensor")
+    for t in (token, seq, count, pos):
+        _check(t is None or (t.is_cuda and t.is_contiguous() and t.dtype == torch.int64 and t.numel() >= 1),
+               "token, seq, count and pos must be int64 CUDA tensors")
+    _check((seq is None) == (count is None), "seq and count go together")
+    _check(workspace.is_cuda and workspace.numel() * workspace.element_size() >= int(_lib.load().decdec_greedy_pick_workspace_bytes()),
+           "workspace too small")
+    _check(logits_f32_out is None or (logits_f32_out.is_cuda and logits_f32_out.is_contiguous() and
+                                      logits_f32_out.dtype == torch.float32 and logits_f32_out.numel() >= logits.numel()),
+           "logits_f32_out must be a contiguous fp32 CUDA tensor of at least as many elements")
+    opt = lambda t: _ptr(t) if t is not None else None
+    _lib.check(_lib.load().decdec_greedy_pick(_ptr(logits), logits.numel(), _dt(logits), _ptr(workspace), opt(logits_f32_out),
+                                              _ptr(token), opt(seq), seq.numel() if seq is not None else 0, opt(count),
+                                              opt(pos), _stream()))

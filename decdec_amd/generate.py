@@ -20,7 +20,7 @@ import time
 
 import torch
 
-from . import _lib, artifacts
+from . import _lib, artifacts, decode_ops
 from .linear import APLinear, LUTGEMMLinear, SQLLMLinear
 from .model import DEC_MODULE_KEYS, Transformer
 
@@ -101,19 +101,26 @@ class DecodeStep:
     """One greedy decode step on static buffers: logits of `token` at `pos`, argmax, the new token appended
     to `seq`, fed back into `token`, `pos` advanced.  `capture()` records it in a HIP graph."""
 
-    def __init__(self, model: Transformer, max_tokens: int):
+    def __init__(self, model: Transformer, max_tokens: int, keep_logits: bool = False):
         dev = model.tok_embeddings.weight.device
         self.model = model
         self.token = torch.zeros(1, 1, dtype=torch.int64, device=dev)
         self.pos = torch.zeros(1, dtype=torch.int64, device=dev)
         self.seq = torch.zeros(max_tokens, dtype=torch.int64, device=dev)
         self.count = torch.zeros(1, dtype=torch.int64, device=dev)
-        self.logits = torch.zeros(1, model.config.vocab_size, dtype=torch.float32, device=dev)
+        self.logits = torch.zeros(1, model.config.vocab_size, dtype=torch.float32, device=dev) if keep_logits else None
+        self.pick_workspace = decode_ops.greedy_pick_workspace(dev) if model.decode_kernels and dev.type == "cuda" else None
         self.graph = None
 
     def _step(self):
         logits = self.model(self.token, self.pos)[:, -1]
-        self.logits.copy_(logits)
+        if self.pick_workspace is not None and logits.dtype in (torch.float16, torch.bfloat16, torch.float32):
+            # argmax and the bookkeeping below in two small launches
+            decode_ops.greedy_pick(logits.contiguous(), self.pick_workspace, self.token, self.seq, self.count, self.pos,
+                                   self.logits)
+            return
+        if self.logits is not None:
+            self.logits.copy_(logits)
         nxt = torch.argmax(logits, dim=-1, keepdim=True)
         self.seq.index_copy_(0, self.count, nxt.view(1))
         self.token.copy_(nxt)

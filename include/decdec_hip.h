@@ -163,7 +163,13 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     are shared by 8 workgroups and a second small kernel merges them; workspace NULL = one workgroup per head.
  *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n.
  *   decdec_add_rmsnorm: per row of `dim` elements (a multiple of 4, <= 16384; 8-byte aligned tensors), h = x + y rounded to the storage type and written to
- *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight. */
+ *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight.
+ *   decdec_greedy_pick: the end of a greedy decode step in two small launches.  token[0] = index of the largest of
+ *     the `n` logits (fp16, bf16 or fp32; the smallest index among equal ones; a NaN with the sign bit clear counts
+ *     as the largest, as in torch.argmax); if seq and count are given, seq[count[0]] = that index (when count[0] <
+ *     seq_capacity) and count[0] += 1; if pos is given, pos[0] += 1; if logits_f32_out is given it receives the
+ *     logits as fp32.  token, seq, count and pos are int64 in device memory; workspace is
+ *     decdec_greedy_pick_workspace_bytes() bytes of 8-byte aligned device memory (contents irrelevant). */
 int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void* sin_table,
                              const int64_t* pos_device, void* q_out, void* k_cache, void* v_cache,
                              int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
@@ -176,6 +182,10 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
 int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
                        int dtype, uint32_t rows, uint32_t dim, float eps, void* stream);
+uint64_t decdec_greedy_pick_workspace_bytes(void);
+int decdec_greedy_pick(const void* logits, uint32_t n, int dtype, void* workspace, float* logits_f32_out,
+                       int64_t* token, int64_t* seq, uint32_t seq_capacity, int64_t* count, int64_t* pos,
+                       void* stream);
 
 /* Diagnostics: with option "dec_trace" = 1 every DEC workgroup stores shader-clock stamps of its
  * phases (0 start, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a

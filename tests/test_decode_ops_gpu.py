@@ -128,3 +128,44 @@ def test_decode_step_on_helper_kernels_equals_the_torch_path():
                   for i, t in enumerate((3, 99, 250))]
         outs[use] = torch.stack(ys)
     assert _close(outs[True], outs[False], 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_greedy_pick_matches_argmax_and_keeps_the_books(dtype):
+    ws = D.greedy_pick_workspace()
+    g = torch.Generator().manual_seed(5)
+    for n in (1, 7, 255, 4097, 32000, 128256):
+        logits = torch.randn(n, generator=g).to(dtype).cuda()
+        token = torch.full((1, 1), -1, dtype=torch.int64, device="cuda")
+        seq = torch.full((4,), -1, dtype=torch.int64, device="cuda")
+        count = torch.tensor([2], dtype=torch.int64, device="cuda")
+        pos = torch.tensor([41], dtype=torch.int64, device="cuda")
+        copy = torch.zeros(n, dtype=torch.float32, device="cuda")
+        D.greedy_pick(logits, ws, token, seq, count, pos, copy)
+        torch.cuda.synchronize()
+        want = int(torch.argmax(logits.float()))
+        assert float(logits[int(token)]) == float(logits[want])           # equal logits: any of them for torch
+        assert int(token) == int((logits == logits[want]).nonzero()[0])   # the smallest index here
+        assert seq.tolist() == [-1, -1, int(token), -1] and int(count) == 3 and int(pos) == 42
+        assert torch.equal(copy, logits.float())
+    # ties, a full sequence buffer, a NaN, optional arguments left out
+    logits = torch.zeros(1000, dtype=dtype, device="cuda")
+    logits[[17, 400, 999]] = 3.0
+    token = torch.zeros(1, dtype=torch.int64, device="cuda")
+    seq = torch.full((2,), -1, dtype=torch.int64, device="cuda")
+    count = torch.tensor([2], dtype=torch.int64, device="cuda")
+    D.greedy_pick(logits, ws, token, seq, count)
+    torch.cuda.synchronize()
+    assert int(token) == 17 and seq.tolist() == [-1, -1] and int(count) == 3
+    logits[500] = float("nan")
+    D.greedy_pick(logits, ws, token)
+    torch.cuda.synchronize()
+    assert int(token) == 500 == int(torch.argmax(logits))
+    logits = -torch.rand(300, device="cuda").to(dtype) - 1.0          # all negative
+    D.greedy_pick(logits, ws, token)
+    torch.cuda.synchronize()
+    assert int(token) == int((logits == logits.max()).nonzero()[0])
+    with pytest.raises(RuntimeError):
+        D.greedy_pick(logits, ws, token, seq)                        # seq without count
+    with pytest.raises(RuntimeError):
+        D.greedy_pick(logits, ws, token.int())

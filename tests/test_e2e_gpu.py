@@ -68,7 +68,7 @@ def test_graph_replays_equal_eager_steps():
     model, _ = _tiny("sqllm", 4)
     with torch.no_grad():
         model(torch.randint(0, model.config.vocab_size, (1, 16), device="cuda"), torch.arange(16, device="cuda"))
-    step = G.DecodeStep(model, max_tokens=16)
+    step = G.DecodeStep(model, max_tokens=16, keep_logits=True)
     step.start(3, 16)
     step.capture()
     for it, (tok, pos) in enumerate([(3, 16), (11, 17), (5, 18), (3, 16)]):
