@@ -958,7 +958,31 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
         }
     }
     AttentionParams p{q, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
-                      1.0f / std::sqrt((float)head_dim), nsplit, (float*)workspace};
+                      1.0f / std::sqrt((float)head_dim), nsplit, (float*)workspace, nullptr, nullptr, nullptr};
+    DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
+    return kOk;
+}
+
+int decdec_rope_attention(const void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos_device,
+                          void* out, void* k_cache, void* v_cache, int dtype, uint32_t n_head, uint32_t n_kv_head,
+                          uint32_t head_dim, uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(qkv && cos_table && sin_table && k_cache && v_cache && pos_device && out, "null pointer argument");
+    DD_CHECK(n_head >= 1 && n_kv_head >= 1 && n_head % n_kv_head == 0, "n_head must be a multiple of n_kv_head");
+    DD_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128, got %u", head_dim);
+    DD_CHECK(max_seq >= 1, "max_seq must be positive");
+    DD_CHECK(((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 && ((uintptr_t)qkv % 16) == 0 &&
+             ((uintptr_t)cos_table % 16) == 0 && ((uintptr_t)sin_table % 16) == 0,
+             "qkv, the tables and the caches must be 16-byte aligned");
+    uint32_t nsplit = 1;
+    if (workspace != nullptr && max_seq > 256) {
+        DD_CHECK(((uintptr_t)workspace % 4) == 0, "workspace must be 4-byte aligned");
+        for (uint32_t n = 8; n > 1; n /= 2) {
+            if (decdec_decode_attention_workspace_bytes(n_head, head_dim, n) <= workspace_bytes) { nsplit = n; break; }
+        }
+    }
+    AttentionParams p{nullptr, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
+                      1.0f / std::sqrt((float)head_dim), nsplit, (float*)workspace, qkv, cos_table, sin_table};
     DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
     return kOk;
 }

@@ -7,6 +7,12 @@
 
 namespace decdec {
 
+// One element of a rotated pair: x c - partner s for the first element of the pair, x c + partner s for the second.
+__device__ __forceinline__ float rope_rotate(float x, float partner, float c, float s, bool first) {
+    const float ps = __fmul_rn(partner, s);
+    return __builtin_fmaf(x, c, first ? -ps : ps);
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void rope_cache_kernel(const RopeCacheParams p) {
     using E = Elem<DT>;
@@ -20,7 +26,7 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const RopeCacheParams p
         const uint32_t head = t / half, i = t % half;
         const float x1 = E::load(p.qkv, (size_t)head * D + i), x2 = E::load(p.qkv, (size_t)head * D + i + half);
         const float c = E::load(p.cos_table, (size_t)pos * D + i), s = E::load(p.sin_table, (size_t)pos * D + i);
-        const float y1 = x1 * c - x2 * s, y2 = x2 * c + x1 * s;
+        const float y1 = rope_rotate(x1, x2, c, s, true), y2 = rope_rotate(x2, x1, c, s, false);
         if (head < p.n_head) {
             E::store(p.q_out, (size_t)head * D + i, y1);
             E::store(p.q_out, (size_t)head * D + i + half, y2);
@@ -73,10 +79,48 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
     const uint16_t* kc = (const uint16_t*)p.k_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
     const uint16_t* vc = (const uint16_t*)p.v_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
     long long pos64 = *p.pos;
-    uint32_t qr[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) qr[e] = *(const uint32_t*)((const uint16_t*)p.q + (size_t)h * D + 8 * dl + 2 * e);
+    const bool fused = p.qkv != nullptr;
+    const bool in_cache = pos64 >= 0 && pos64 < (long long)p.max_seq;      // the new token has a cache row
     if (pos64 < 0) pos64 = 0;
+    uint32_t qr[4];
+    u32x4 knew = {0u, 0u, 0u, 0u}, vnew = {0u, 0u, 0u, 0u};
+    const uint32_t newpos = (fused && in_cache) ? (uint32_t)pos64 : 0xFFFFFFFFu;
+    if (fused) {
+        // the lane's eight elements start at 8 dl; their rotation partners sit half a head away; the tables hold
+        // the angle of pair i at [pos][i], i < D / 2 (a position past the tables uses their last row)
+        constexpr uint32_t half = D / 2;
+        const uint32_t e0 = 8u * dl, pe0 = (e0 + half) % (uint32_t)D, te0 = e0 % half;
+        const bool first = e0 < half;
+        const size_t trow = (size_t)((pos64 < (long long)p.max_seq) ? pos64 : (long long)p.max_seq - 1) * D;
+        const u32x4 cr = *(const u32x4*)((const uint16_t*)p.cos_table + trow + te0);
+        const u32x4 sr = *(const u32x4*)((const uint16_t*)p.sin_table + trow + te0);
+        const uint16_t* qh = (const uint16_t*)p.qkv + (size_t)h * D;
+        const uint16_t* kh = (const uint16_t*)p.qkv + (size_t)(p.n_head + kvh) * D;
+        const u32x4 qs = *(const u32x4*)(qh + e0), qp = *(const u32x4*)(qh + pe0);
+        const u32x4 ks = *(const u32x4*)(kh + e0), kp = *(const u32x4*)(kh + pe0);
+        vnew = *(const u32x4*)((const uint16_t*)p.qkv + (size_t)(p.n_head + p.n_kv + kvh) * D + e0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            uint32_t qo = 0u, ko = 0u;
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf) {
+                const int sh = 16 * hf;
+                const float c = E::from_raw((cr[e] >> sh) & 0xFFFFu), sn = E::from_raw((sr[e] >> sh) & 0xFFFFu);
+                const float xq = E::from_raw((qs[e] >> sh) & 0xFFFFu), pq = E::from_raw((qp[e] >> sh) & 0xFFFFu);
+                const float xk = E::from_raw((ks[e] >> sh) & 0xFFFFu), pk = E::from_raw((kp[e] >> sh) & 0xFFFFu);
+                // first half: x c - partner s; second half: x c + partner s, rounded to the storage type as a
+                // separate rotary kernel stores them (the compiler may round a near-tie the other way here)
+                const float yq = rope_rotate(xq, pq, c, sn, first), yk = rope_rotate(xk, pk, c, sn, first);
+                qo |= (E::to_raw(yq) & 0xFFFFu) << sh;
+                ko |= (E::to_raw(yk) & 0xFFFFu) << sh;
+            }
+            qr[e] = qo;
+            knew[e] = ko;
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qr[e] = *(const uint32_t*)((const uint16_t*)p.q + (size_t)h * D + 8 * dl + 2 * e);
+    }
     const uint32_t len = (uint32_t)((pos64 + 1 < (long long)p.max_seq) ? pos64 + 1 : (long long)p.max_seq);
     // this workgroup's positions: [lo, hi), ranges of a multiple of 16 PPW positions
     const uint32_t chunk = ((len + nsplit - 1u) / nsplit + 16u * PPW - 1u) / (16u * PPW) * (16u * PPW);
@@ -99,6 +143,7 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
             const uint32_t ppc = pp < hi ? pp : hi - 1u;
             kr[u] = *(const u32x4*)(kc + (size_t)ppc * D);
             vr[u] = *(const u32x4*)(vc + (size_t)ppc * D);
+            if (ppc == newpos) { kr[u] = knew; vr[u] = vnew; }             // the new token's row is not in the cache yet
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -122,6 +167,11 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
                 m = mn;
             }
         }
+    }
+    // cache append: one workgroup per key/value head (its first query head, the range that holds the position)
+    if (newpos != 0xFFFFFFFFu && h % (p.n_head / p.n_kv) == 0u && newpos >= lo && newpos < hi && tid < (uint32_t)LPP) {
+        *(u32x4*)((uint16_t*)p.k_cache + ((size_t)kvh * p.max_seq + newpos) * D + 8 * dl) = knew;
+        *(u32x4*)((uint16_t*)p.v_cache + ((size_t)kvh * p.max_seq + newpos) * D + 8 * dl) = vnew;
     }
     const uint32_t g = wave * PPW + sub;
     if (dl == 0) { pm[g] = m; pl[g] = l; }

@@ -64,6 +64,12 @@ struct AttentionParams {
     float scale;
     uint32_t nsplit;                 // workgroups per head (1: no workspace needed)
     float* workspace;                // [n_head][nsplit][head_dim + 2] floats
+    // Rotary embedding and cache append folded in (qkv != null; q is not read then): queries and the new key are
+    // rotated on the fly, the new key / value row takes the place of cache row *pos in the scan, and the first
+    // query head of every key/value head writes that row to the caches.
+    const void* qkv;                 // [(n_head + 2 n_kv) * head_dim]
+    const void* cos_table;           // [max_seq][head_dim]
+    const void* sin_table;
 };
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);

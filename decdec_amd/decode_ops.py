@@ -49,6 +49,25 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                                                    workspace.numel() * 4 if workspace is not None else 0, _stream()))
 
 
+def rope_attention(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor, pos: torch.Tensor,
+                   out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, n_head: int, n_kv_head: int,
+                   workspace: torch.Tensor | None = None) -> None:
+    """`rope_cache_update` + `decode_attention` in one launch: un-rotated qkv in, attention output out, the new key /
+    value row appended to the caches."""
+    _half_cuda(qkv, cos_table, sin_table, out, k_cache, v_cache)
+    _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64 on the device")
+    D, max_seq = k_cache.shape[-1], k_cache.shape[-2]
+    _check(qkv.numel() == (n_head + 2 * n_kv_head) * D and out.numel() == n_head * D, "qkv / out size mismatch")
+    _check(k_cache.numel() == n_kv_head * max_seq * D and v_cache.shape == k_cache.shape, "cache shape mismatch")
+    _check(tuple(cos_table.shape) == (max_seq, D) and tuple(sin_table.shape) == (max_seq, D), "rotary tables must be [max_seq, head_dim]")
+    if workspace is not None:
+        _check(workspace.is_cuda and workspace.is_contiguous() and workspace.dtype == torch.float32, "workspace must be a contiguous float32 CUDA tensor")
+    _lib.check(_lib.load().decdec_rope_attention(_ptr(qkv), _ptr(cos_table), _ptr(sin_table), _ptr(pos), _ptr(out),
+                                                 _ptr(k_cache), _ptr(v_cache), _dt(qkv), n_head, n_kv_head, D, max_seq,
+                                                 _ptr(workspace) if workspace is not None else None,
+                                                 workspace.numel() * 4 if workspace is not None else 0, _stream()))
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _half_cuda(gate_up, out)
     _check(gate_up.numel() == 2 * out.numel(), "gate_up must hold twice as many elements as out")

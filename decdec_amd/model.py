@@ -125,14 +125,12 @@ class Attention(nn.Module):
         kv = self.n_local_heads * self.head_dim
         qkv = self.wqkv(x)
         if rope_tables_full is not None:
-            # one-token step on the library's helper kernels: rotate + append to the cache, then attend
+            # one-token step on the library's helper kernel: rotate, append to the cache and attend in one launch
             from . import decode_ops
-            q = torch.empty(self.dim, dtype=x.dtype, device=x.device)
-            decode_ops.rope_cache_update(qkv.view(-1), rope_tables_full[0], rope_tables_full[1], input_pos, q,
-                                         self.kv_cache.k_cache, self.kv_cache.v_cache, self.n_head, self.n_local_heads)
             y = torch.empty(1, 1, self.dim, dtype=x.dtype, device=x.device)
-            decode_ops.decode_attention(q, self.kv_cache.k_cache, self.kv_cache.v_cache, input_pos, y,
-                                        self.n_head, self.n_local_heads, rope_tables_full[2])
+            decode_ops.rope_attention(qkv.view(-1), rope_tables_full[0], rope_tables_full[1], input_pos, y,
+                                      self.kv_cache.k_cache, self.kv_cache.v_cache, self.n_head, self.n_local_heads,
+                                      rope_tables_full[2])
             return self.wo(y)
         # RoPE on the query and key heads in one pass (they are neighbours in the fused projection)
         nqk = self.n_head + self.n_local_heads

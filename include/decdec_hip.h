@@ -161,6 +161,12 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     decdec_decode_attention_workspace_bytes(n_head, head_dim, 8) bytes (caller-owned device memory, contents
  *     irrelevant; one workspace serves any number of calls that do not overlap in time) the positions of a head
  *     are shared by 8 workgroups and a second small kernel merges them; workspace NULL = one workgroup per head.
+ *   decdec_rope_attention: the two calls above in one launch (plus the merge kernel when a workspace is given): takes
+ *     the un-rotated qkv, rotates the queries and the new key on the fly (rounded to the storage type; a value
+ *     within rounding error of a tie may differ by one unit in the last place from what decdec_rope_cache_update
+ *     stores), attends cache rows 0 .. pos - 1 and the new row, and appends the new
+ *     key / value row to the caches (position outside [0, max_seq): nothing is appended, rows 0 .. max_seq - 1 are
+ *     attended).  qkv, the tables and the caches 16-byte aligned.
  *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n.
  *   decdec_add_rmsnorm: per row of `dim` elements (a multiple of 4, <= 16384; 8-byte aligned tensors), h = x + y rounded to the storage type and written to
  *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight.
@@ -179,6 +185,10 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
                             const int64_t* pos_device, void* out, int dtype, uint32_t n_head,
                             uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq,
                             void* workspace, uint64_t workspace_bytes, void* stream);
+int decdec_rope_attention(const void* qkv, const void* cos_table, const void* sin_table,
+                          const int64_t* pos_device, void* out, void* k_cache, void* v_cache, int dtype,
+                          uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq,
+                          void* workspace, uint64_t workspace_bytes, void* stream);
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
 int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
                        int dtype, uint32_t rows, uint32_t dim, float eps, void* stream);

@@ -71,6 +71,54 @@ def test_decode_attention(H, Hkv, hd, S, dt):
     assert torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,hd,S", [(8, 2, 64, 256), (32, 8, 128, 2048), (4, 4, 128, 80), (40, 10, 128, 520)])
+def test_rope_attention_equals_the_two_step_form(H, Hkv, hd, S, dt):
+    """One launch for rotary embedding + cache append + attention against rope_cache_update followed by
+    decode_attention (with and without the workspace) and against fp32 torch: same values row and same output to
+    within rounding (a rotated value that sits within fp32 rounding error of a 16-bit tie may be rounded either
+    way by either kernel), nothing but the new row touched."""
+    g = torch.Generator(device="cuda").manual_seed(2)
+    cos, sin = rope_tables(hd, S, 10000.0, "cuda")
+    cos16, sin16 = cos.to(dt), sin.to(dt)
+    kc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    vc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").to(dt)
+    ws = D.attention_workspace(H, hd)
+    for pos in sorted({0, 1, 15, 16, 63, 64, S // 2 + 3, S - 1}):
+        qkv = (torch.randn((H + 2 * Hkv) * hd, generator=g, device="cuda") * 1.5).to(dt)
+        p = torch.tensor([pos], device="cuda")
+        k2, v2 = kc.clone(), vc.clone()
+        q_rot = torch.empty(H * hd, dtype=dt, device="cuda")
+        want = torch.empty(H * hd, dtype=dt, device="cuda")
+        D.rope_cache_update(qkv, cos16, sin16, p, q_rot, k2, v2, H, Hkv)
+        D.decode_attention(q_rot, k2, v2, p, want, H, Hkv)
+        for w in (None, ws):
+            k1, v1 = kc.clone(), vc.clone()
+            out = torch.empty(H * hd, dtype=dt, device="cuda")
+            D.rope_attention(qkv, cos16, sin16, p, out, k1, v1, H, Hkv, w)
+            torch.cuda.synchronize()
+            assert torch.equal(v1, v2), (pos, w is not None)
+            keep = torch.ones(S, dtype=torch.bool, device="cuda"); keep[pos] = False
+            assert torch.equal(k1[0][:, keep], kc[0][:, keep]), pos
+            ulp = 2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10       # one unit in the last place, relative
+            assert float(((k1 - k2).float().abs() / k2.float().abs().clamp_min(1e-3)).max()) <= ulp, pos
+            assert int((k1 != k2).sum()) <= 4, pos
+            assert _close(out, want, 2e-2 if dt == torch.bfloat16 else 3e-3), pos
+        # fp32 torch on the rotated query and the updated cache
+        k = k2[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)
+        v = v2[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)
+        att = torch.softmax(torch.einsum("hd,hld->hl", q_rot.float().view(H, hd), k) / math.sqrt(hd), dim=-1)
+        ref = torch.einsum("hl,hld->hd", att, v)
+        assert _close(out.view(H, hd), ref, 2e-2 if dt == torch.bfloat16 else 3e-3), pos
+        kc, vc = k2, v2                                         # keep appending
+    # a position outside the cache appends nothing and reads nothing outside it
+    k0, v0 = kc.clone(), vc.clone()
+    for bad in (-1, S, S + 100):
+        D.rope_attention(qkv, cos16, sin16, torch.tensor([bad], device="cuda"), out, kc, vc, H, Hkv, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, k0) and torch.equal(vc, v0) and torch.isfinite(out.float()).all()
+
+
 @pytest.mark.parametrize("n", [1, 255, 14336])
 def test_silu_mul(n):
     gu = torch.randn(2 * n, device="cuda").half() * 3
