@@ -408,8 +408,12 @@ __device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bi
     if constexpr (BITS == 3) {
         if (p.tile_cs != 0u) { anyprec3_tile<DT>(p, bid, smem); return; }
     }
-    if (p.rpw == 8) anyprec_rows<DT, BITS, 8>(p, bid, smem);
-    else if (p.rpw == 4) anyprec_rows<DT, BITS, 4>(p, bid, smem);
+    // eight rows per wave only at 3 bits: the plane words of eight rows of a wider format do not fit the register
+    // budget (the launch planner never asks for it)
+    if constexpr (BITS == 3) {
+        if (p.rpw == 8) { anyprec_rows<DT, BITS, 8>(p, bid, smem); return; }
+    }
+    if (p.rpw >= 4) anyprec_rows<DT, BITS, 4>(p, bid, smem);
     else anyprec_rows<DT, BITS, 2>(p, bid, smem);
 }
 

@@ -362,6 +362,7 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     uint32_t rpw = row_slices >= 32768 ? 8u : (row_slices >= 8192 ? 4u : 2u);
     if (row_slices >= 16384 && p.S * p.sgroups >= 4) rpw = 8u;     // long rows (K >= 8192): measured 9.0 against 10.1 us at 14336 -> 4096
     if (g_opt.anyprec_rpw == 2 || g_opt.anyprec_rpw == 4 || g_opt.anyprec_rpw == 8) rpw = (uint32_t)g_opt.anyprec_rpw;
+    if (bits > 3) rpw = std::min(rpw, 4u);      // wider formats: four rows of plane words per wave fit the registers, eight do not
     p.rpw = rpw;
     if (g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
     p.x_aligned = ((uintptr_t)input % 16) == 0;
