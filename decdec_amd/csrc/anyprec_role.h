@@ -133,6 +133,48 @@ __device__ __forceinline__ void anyprec3_tables(const u32x4 lut4, uint32_t& lo0,
     hi1 = __builtin_amdgcn_perm(lut4[3], lut4[2], 0x07050301u);
 }
 
+// One word of a 4-bit row, same scheme with 16-entry tables: the low three index bits select inside a table half
+// (entries 0..7 in LO[0..1] / HI[0..1], 8..15 in LO[2..3] / HI[2..3]), the fourth picks the half bytewise.
+struct Anyprec4Masks {
+    uint32_t m8, m4, m2, k7, k1;
+    __device__ __forceinline__ void init() {
+        m8 = 0x88888888u; m4 = 0x44444444u; m2 = 0x22222222u; k7 = 0x07070707u; k1 = 0x01010101u;
+        asm volatile("" : "+v"(m8), "+v"(m4), "+v"(m2), "+v"(k7), "+v"(k1));
+    }
+};
+template <int DT>
+__device__ __forceinline__ float anyprec4_word(uint32_t q0, uint32_t q1, uint32_t q2, uint32_t q3,
+                                               const uint32_t (&lo)[4], const uint32_t (&hi)[4], const Anyprec4Masks& mk,
+                                               const uint32_t (&xp)[8][2], float acc) {
+    // index words: nibble n of T_o carries the 4-bit index of bit 4n+o (plane 0 = most significant bit)
+    const uint32_t t3 = bit_select(mk.m8, q0, bit_select(mk.m4, q1 >> 1, bit_select(mk.m2, q2 >> 2, q3 >> 3)));
+    const uint32_t t2 = bit_select(mk.m8, q0 << 1, bit_select(mk.m4, q1, bit_select(mk.m2, q2 >> 1, q3 >> 2)));
+    const uint32_t t1 = bit_select(mk.m8, q0 << 2, bit_select(mk.m4, q1 << 1, bit_select(mk.m2, q2, q3 >> 1)));
+    const uint32_t t0 = bit_select(mk.m8, q0 << 3, bit_select(mk.m4, q1 << 2, bit_select(mk.m2, q2 << 1, q3)));
+    const uint32_t tt[4] = {t3, t2, t1, t0};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        // selector bytes 0..3 <-> j = 3..0; e < 4: the upper nibbles of T_(3-e), e >= 4: the lower nibbles of T_(7-e)
+        const uint32_t t = (e < 4) ? (tt[e] >> 4) : tt[e - 4];
+        const uint32_t sel = t & mk.k7;
+        const uint32_t half = ((t >> 3) & mk.k1) * 255u;                    // 0xFF in the bytes whose index is >= 8
+        const uint32_t L = bit_select(half, __builtin_amdgcn_perm(lo[3], lo[2], sel), __builtin_amdgcn_perm(lo[1], lo[0], sel));
+        const uint32_t H = bit_select(half, __builtin_amdgcn_perm(hi[3], hi[2], sel), __builtin_amdgcn_perm(hi[1], hi[0], sel));
+        const uint32_t w32 = __builtin_amdgcn_perm(H, L, 0x05010400u);   // weights j3, j2
+        const uint32_t w10 = __builtin_amdgcn_perm(H, L, 0x07030602u);   // weights j1, j0
+        acc = dot2_acc<DT>(w32, xp[e][0], acc);
+        acc = dot2_acc<DT>(w10, xp[e][1], acc);
+    }
+    return acc;
+}
+// byte tables of a row's sixteen 16-bit LUT entries (two per dword)
+__device__ __forceinline__ void anyprec4_tables(const u32x4 a, const u32x4 b, uint32_t (&lo)[4], uint32_t (&hi)[4]) {
+    lo[0] = __builtin_amdgcn_perm(a[1], a[0], 0x06040200u); hi[0] = __builtin_amdgcn_perm(a[1], a[0], 0x07050301u);
+    lo[1] = __builtin_amdgcn_perm(a[3], a[2], 0x06040200u); hi[1] = __builtin_amdgcn_perm(a[3], a[2], 0x07050301u);
+    lo[2] = __builtin_amdgcn_perm(b[1], b[0], 0x06040200u); hi[2] = __builtin_amdgcn_perm(b[1], b[0], 0x07050301u);
+    lo[3] = __builtin_amdgcn_perm(b[3], b[2], 0x06040200u); hi[3] = __builtin_amdgcn_perm(b[3], b[2], 0x07050301u);
+}
+
 // Generic bit width: indices assembled bytewise, weights from a per-wave LDS copy of the LUT (fp32).
 template <int DT, int BITS>
 __device__ __forceinline__ float anyprec_generic_word(const uint32_t (&q)[BITS], const float* wlut,
@@ -236,12 +278,19 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
         uint32_t xr[4][4];
         anyprec_issue_x(p, wi_c, xr);
         const uint32_t word_off = wi_c * 4u;        // byte offset of the lane's word inside a row
-        u32x4 lut4[RB];
+        u32x4 lut4[RB], lut4b[RB];
         if constexpr (BITS == 3) {
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
                 const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
                 lut4[r] = *(const DD_CONST_AS u32x4*)((const uint16_t*)p.lut + (size_t)row * 8);
+            }
+        } else if constexpr (BITS == 4) {
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
+                lut4[r] = *(const DD_CONST_AS u32x4*)((const uint16_t*)p.lut + (size_t)row * 16);
+                lut4b[r] = *(const DD_CONST_AS u32x4*)((const uint16_t*)p.lut + (size_t)row * 16 + 8);
             }
         }
         // unconditional loads from wave-uniform row bases (rows past the end re-read the last row)
@@ -259,7 +308,8 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
         anyprec_arrange_x(xr, xp);
         float sums[RB];
         Anyprec3Masks mk;
-        mk.init();
+        Anyprec4Masks mk4;
+        if constexpr (BITS == 4) mk4.init(); else mk.init();
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
             float acc;
@@ -267,6 +317,10 @@ __device__ __forceinline__ void anyprec_rows(const AnyprecParams& p, uint32_t bi
                 uint32_t lo0, lo1, hi0, hi1;
                 anyprec3_tables(lut4[r], lo0, lo1, hi0, hi1);
                 acc = anyprec3_word<DT>(q[r][0], q[r][1], q[r][2], lo0, lo1, hi0, hi1, mk, xp, 0.f);
+            } else if constexpr (BITS == 4) {
+                uint32_t lo[4], hi[4];
+                anyprec4_tables(lut4[r], lut4b[r], lo, hi);
+                acc = anyprec4_word<DT>(q[r][0], q[r][1], q[r][2], q[r][3], lo, hi, mk4, xp, 0.f);
             } else {
                 constexpr int L = 1 << BITS;
                 const uint32_t row = ((uint32_t)r < nrows) ? row0 + r : (p.N - 1u);
@@ -408,8 +462,8 @@ __device__ __forceinline__ void anyprec_role(const AnyprecParams& p, uint32_t bi
     if constexpr (BITS == 3) {
         if (p.tile_cs != 0u) { anyprec3_tile<DT>(p, bid, smem); return; }
     }
-    // eight rows per wave only at 3 bits: the plane words of eight rows of a wider format do not fit the register
-    // budget (the launch planner never asks for it)
+    // eight rows per wave only at 3 bits: the plane words of eight rows of a wider format cost occupancy (4 bits:
+    // 82 registers against 65) or do not fit the register budget at all (the launch planner never asks for it)
     if constexpr (BITS == 3) {
         if (p.rpw == 8) { anyprec_rows<DT, BITS, 8>(p, bid, smem); return; }
     }

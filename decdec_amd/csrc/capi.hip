@@ -345,7 +345,7 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     DD_CHECK(input && output && qweight && lut, "null pointer argument");
     DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
     DD_CHECK(N >= 1, "output_feat must be positive");
-    DD_CHECK(((uintptr_t)lut % 16) == 0 || bits != 3, "lut must be 16-byte aligned");
+    DD_CHECK(((uintptr_t)lut % 16) == 0 || bits > 4, "lut must be 16-byte aligned");
     DD_CHECK(((uintptr_t)output % 4) == 0, "output must be 4-byte aligned");
     AnyprecParams& p = pl->p;
     memset(&p, 0, sizeof(p));
