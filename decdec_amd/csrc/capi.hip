@@ -337,7 +337,7 @@ int check_dec_call(const Config* c, int dtype, uint32_t in_features, uint32_t ou
 struct AnyprecPlan { AnyprecParams p; LaunchDims d; };
 
 int plan_anyprec(const void* input, void* output, const void* qweight, const void* lut, int bits, int dtype,
-                 uint32_t K, uint32_t N, bool fused_block, AnyprecPlan* pl) {
+                 uint32_t K, uint32_t N, bool fused_block, AnyprecPlan* pl, uint32_t rpw_cap = 8) {
     DD_CHECK(bits >= 3 && bits <= 8, "Bitwidth must be between 3 and 8.");
     if (dtype == DECDEC_FP32)
         return fail(kUnsupported, "Any-Precision GEMV does not support float data type. Please use half or bfloat16.");
@@ -363,6 +363,7 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     if (row_slices >= 16384 && p.S * p.sgroups >= 4) rpw = 8u;     // long rows (K >= 8192): measured 9.0 against 10.1 us at 14336 -> 4096
     if (g_opt.anyprec_rpw == 2 || g_opt.anyprec_rpw == 4 || g_opt.anyprec_rpw == 8) rpw = (uint32_t)g_opt.anyprec_rpw;
     if (bits > 3) rpw = std::min(rpw, 4u);      // wider formats: four rows of plane words per wave fit the registers, eight do not
+    if (g_opt.anyprec_rpw == 0) rpw = std::min(rpw, rpw_cap);
     p.rpw = rpw;
     if (g_opt.anyprec_rg > 0) p.rg = std::min((uint32_t)g_opt.anyprec_rg, std::max(1u, 16u / p.S));
     p.x_aligned = ((uintptr_t)input % 16) == 0;
@@ -817,7 +818,10 @@ int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* 
     if (fuse && bits == 3 && g_opt.fused_small != 0) {
         // Both roles in workgroups of the GEMV's own size (4 or 8 waves): the GEMV keeps its standalone
         // schedule and a DEC workgroup holds an eighth or a quarter of a compute unit instead of a half.
-        rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, false, &pl);
+        // four rows per wave: beside DEC workgroups twice as many, shorter GEMV workgroups measured 1 us faster
+        // (14336 -> 4096: 11.0 / 11.4 / 13.5 us against 12.0 / 12.6 / 14.6 us at k_chunk 1 / 4 / 8) although the
+        // GEMV alone is slower that way (10.2 against 9.6 us)
+        rc = plan_anyprec(input, output, qweight, lut, bits, dtype, K, N, false, &pl, 4u);
         if (rc != kOk) return rc;
         const uint32_t nw = pl.d.block <= 256u ? 4u : (pl.d.block <= 512u ? 8u : 16u);
         if (pl.p.tile_cs == 0u && fused_small(c, (double)bits * N * K / 8.0, nw)) {
