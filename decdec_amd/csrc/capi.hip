@@ -795,12 +795,15 @@ bool fused_two_per_cu(const Config* c, double gemv_bytes) {
 // size).  Measured at 14336 -> 4096 (8 waves): 12.0 / 12.6 / 14.6 us against 13.3 / 16.4 / 15.9 us for the
 // 1024-thread form at k_chunk 1 / 4 / 8, but 16.7 against 15.9 us at k_chunk 12 and 26.5 against 24.0 us at 32: a
 // DEC workgroup's host-memory reads hold up the GEMV waves of its compute unit, and the small form spreads the DEC
-// workgroups over four times as many units, so it only pays while the GEMV is the longer role.  With 4-wave
-// workgroups (K <= 8192) the 1024-thread form was as fast or faster at every k_chunk.
+// workgroups over four times as many units, so it only pays while the GEMV is the longer role.  Inside a decode step
+// (14336 -> 4096, cost over the GEMV per launch) the small form measured 1.3 / 3.5 / 4.4 / 5.5 / 7.5 us at k_chunk
+// 4 / 8 / 10 / 12 / 16 against 6.6 / 6.4 / 6.4 / 6.4 / 7.1 us: the switch sits where DEC is estimated at 1.4 x the
+// GEMV (k_chunk 14 there).  With 4-wave workgroups (K <= 8192) the 1024-thread form was as fast or faster at every
+// k_chunk.
 bool fused_small(const Config* c, double gemv_bytes, uint32_t nw) {
     if (nw >= 16u || g_opt.fused_small == 0) return false;
     if (g_opt.fused_small > 0) return true;
-    return nw == 8u && dec_estimate_us(c) < 1.2 * gemv_estimate_us(gemv_bytes);
+    return nw == 8u && dec_estimate_us(c) < 1.4 * gemv_estimate_us(gemv_bytes);
 }
 
 int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
