@@ -37,6 +37,16 @@ def test_version_and_options():
     _lib.set_option("fusion", 1)
     with pytest.raises(RuntimeError, match="unknown option"):
         _lib.set_option("no_such_option", 1)
+    # every option the header names exists, with the documented default
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "decdec_hip.h")).read()
+    block = header[header.index("/* Library options:"):header.index("int decdec_set_option")]
+    named = set(re.findall(r'"([a-z0-9_]+)"', block))
+    defaults = {"fusion": 1, "host_noncoherent": 0, "anyprec_rpw": 0, "anyprec_tile": 0, "lutgemm_ktiles": 0,
+                "sqllm_ktiles": 0, "fused_two_per_cu": -1, "fused_small": -1, "anyprec_rg": 0, "dec_block_waves": 16,
+                "dec_trace": 0}
+    assert named == set(defaults), named ^ set(defaults)
+    for name, value in defaults.items():
+        assert _lib.get_option(name) == value, name
 
 
 @pytest.mark.parametrize("dt,code", [("fp16", 1), ("bf16", 2), ("fp32", 0)])
