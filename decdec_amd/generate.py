@@ -63,6 +63,7 @@ def init_random_weights(model: Transformer, seed: int = 0, std: float = 0.02) ->
 def calibrate_thresholds(model: Transformer, seq_len: int = 256, passes: int = 2, seed: int = 1):
     """Thresholds of the four compensated linears of every layer from prefill passes over random tokens."""
     dev = model.tok_embeddings.weight.device
+    seq_len = min(seq_len, model.max_seq_length)          # positions beyond the cache would index outside the mask
     gen = torch.Generator(device=dev).manual_seed(seed)
     named = [(f"layers.{i}.{key}", lin) for i, layer in enumerate(model.layers)
              for key, lin in zip(DEC_MODULE_KEYS, layer.dec_linears())]

@@ -259,6 +259,8 @@ class Transformer(nn.Module):
     def forward(self, idx: torch.Tensor, input_pos: torch.Tensor) -> torch.Tensor:
         """idx [B, S] token ids, input_pos [S] positions (int64); returns logits [B, S, vocab]."""
         assert self.max_seq_length > 0, "Caches must be initialized first"
+        assert idx.shape[1] <= self.max_seq_length and input_pos.numel() == idx.shape[1], \
+            f"{idx.shape[1]} positions do not fit a cache of {self.max_seq_length} (input_pos must hold one position per token)"
         if idx.shape[1] == 1 and getattr(self, "output_arena", None) is not None:
             self.output_arena.zero_()
         x = self.tok_embeddings(idx)

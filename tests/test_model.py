@@ -136,3 +136,10 @@ def test_threshold_collector_is_the_running_max_of_sorted_magnitudes():
     want = torch.stack([torch.sort(r, descending=True).values for r in allx]).amax(0)
     assert torch.equal(th, want)
     assert torch.all(th[:-1] >= th[1:])
+
+
+def test_prefill_longer_than_the_cache_is_refused():
+    """More prompt positions than cache rows must fail on the host, not index outside the mask on the device."""
+    model, _ = _dense_model()                       # 64 cache rows
+    with pytest.raises(AssertionError, match="do not fit a cache"):
+        model(torch.zeros(1, 80, dtype=torch.int64), torch.arange(80))
