@@ -1,0 +1,102 @@
+"""Seeded sweeps over irregular shapes: DEC alone and fused with the any-precision GEMV in every launch form, and
+the three base GEMVs at every bit width, group size and dtype, each against the oracle (selection bit-exact,
+outputs within the tolerances of test_gpu_parity)."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from decdec_amd import _lib, ext, formats as F
+from helpers import make_dec_layer, np_of, rel_err
+from oracle import decdec_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"fp16": 1e-2, "bf16": 8e-2, "fp32": 1e-2}
+TORCH = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+def _reset_options():
+    for name, value in (("dec_block_waves", 16), ("fused_small", -1), ("fused_two_per_cu", -1)):
+        _lib.set_option(name, value)
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_dec_and_fused_forms_on_random_shapes(seed, c_oracle):
+    rng = random.Random(seed)
+    for case in range(14):
+        K = rng.choice([1024, 1536, 2048, 3072, 4096, 5120, 8192, 11008]) if rng.random() < 0.7 else 32 * rng.randint(33, 300)
+        N = 8 * rng.randint(1, 400) if rng.random() < 0.5 else rng.choice([1024, 2056, 4096, 6144])
+        kc = rng.choice([1, 2, 3, 4, 8, 16, 32, 64, 100, 200, 256, 300])
+        n_tb = rng.choice([1, 2, 4, 8, 16, 32, 64])
+        dt = rng.choice(["fp16", "bf16"])
+        mode = rng.choice(["dec", "dec4", "dec8", "fused", "fused_small", "fused_two"])
+        L = make_dec_layer(K, N, seed=rng.randint(0, 10 ** 6), dtype=TORCH[dt])
+        chunks = -(-K // 1024)
+        rows = torch.full((chunks * kc + 64,), -7, dtype=torch.int32, device="cuda")
+        acts = torch.zeros(chunks * kc + 64, dtype=TORCH[dt], device="cuda")
+        ctx = ext.create_dec_context(n_tb, rows, acts)
+        cfg = ext.create_dec_config(ctx, kc, L["cheat"], L["scales"], L["th"])
+        out = torch.zeros(1, 1, N, dtype=TORCH[dt], device="cuda")
+        x = L["x"].cuda()
+        base = 0.0
+        try:
+            if mode.startswith("dec"):
+                _lib.set_option("dec_block_waves", int(mode[3:] or 16))
+                ext.dec(cfg, x, out)
+            else:
+                _lib.set_option("fused_small", 1 if mode == "fused_small" else -1)
+                _lib.set_option("fused_two_per_cu", 1 if mode == "fused_two" else -1)
+                ext.dec_anyprec(cfg, x, out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+                base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3, dt)
+            torch.cuda.synchronize()
+        finally:
+            _reset_options()
+        what = (seed, case, K, N, kc, n_tb, dt, mode)
+        want_rows, _, filled = O.select_channels(np_of(L["x"]), np_of(L["th"]), kc, dt)
+        got = rows.cpu().numpy()[: len(want_rows)]
+        assert np.array_equal(got[filled], want_rows[filled]) and (got[~filled] == -7).all(), what
+        want = base + c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows[filled], dt)
+        mre, mae = rel_err(np_of(out).reshape(-1), want)
+        assert mre <= TOL[dt], what + (mre, mae)
+        ext.destroy_dec_config(cfg)
+        ext.destroy_dec_context(ctx)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_base_gemvs_on_random_shapes(seed, c_oracle):
+    rng = random.Random(seed)
+    for case in range(150):
+        kind = rng.choice(["anyprec", "anyprec", "lutgemm", "sqllm"])
+        K = 32 * rng.randint(1, 300) if rng.random() < 0.7 else rng.choice([1024, 4096, 5120, 8192, 11008])
+        N = rng.randint(1, 2000) if rng.random() < 0.7 else rng.choice([1024, 4096, 6144])
+        dt = rng.choice(["fp16", "bf16"] if kind == "anyprec" else ["fp16", "bf16", "fp32"])
+        g = torch.Generator().manual_seed(rng.randint(0, 10 ** 6))
+        x = F.make_activation(K, g, dtype=TORCH[dt])
+        out = torch.zeros(1, 1, N, dtype=TORCH[dt], device="cuda")
+        words = lambda *shape: torch.randint(-2 ** 31, 2 ** 31 - 1, shape, generator=g, dtype=torch.int64).to(torch.int32)
+        if kind == "anyprec":
+            bits = rng.choice([3, 3, 4, 4, 5, 6, 7, 8])
+            qw, lut = words(bits, N, K // 32), (torch.randn(N, 2 ** bits, generator=g) * 0.05).to(TORCH[dt])
+            ext.anyprec_gemv(x.cuda(), out, qw.cuda(), lut.cuda(), bits)
+            want = c_oracle.anyprec_gemv(np_of(x), qw.numpy(), np_of(lut), bits, dt)
+        elif kind == "sqllm":
+            bits = rng.choice([3, 4])
+            if (K * bits) % 32:
+                continue
+            mat, lut = words(K * bits // 32, N), (torch.randn(N, 2 ** bits, generator=g) * 0.05).to(TORCH[dt])
+            ext.sqllm_gemv(x.cuda(), out, mat.cuda(), lut.cuda(), bits)
+            want = c_oracle.sqllm_gemv(np_of(x), mat.numpy(), np_of(lut), bits, dt)
+        else:
+            bits, group = rng.choice([2, 3, 4, 8]), rng.choice([32, 64, 128, 256])
+            if K % group:
+                continue
+            qw = words(K // 32, bits, N)
+            alpha = (torch.rand(K // group, bits, N, generator=g) * 0.02).to(TORCH[dt])
+            qb = (torch.randn(K // group, N, generator=g) * 0.01).to(TORCH[dt])
+            ext.lutgemm_gemv(x.cuda(), out, qw.cuda(), alpha.cuda(), qb.cuda(), bits, group)
+            want = c_oracle.lutgemm_gemv(np_of(x), qw.numpy(), np_of(alpha), np_of(qb), bits, group, dt)
+        torch.cuda.synchronize()
+        mre, mae = rel_err(np_of(out).reshape(-1), want)
+        assert mre <= TOL[dt], (seed, case, kind, K, N, bits, dt, mre, mae)
