@@ -776,19 +776,35 @@ int decdec_sqllm_gemv(const void* input, void* output, const void* mat, const vo
 }
 
 // ---------------------------------------------------------------- DEC + base GEMV
-// Which instance of a fused kernel to launch: the one that lets two workgroups share a compute unit when the
-// GEMV role is expected to outlast the DEC role by a margin.  Estimates in microseconds: DEC = its latency
-// floor (launch, activation load, selection, one host-link round trip, merge: about 8) plus the residual
-// bytes at the zero-copy rate of the link (56 GB/s); GEMV = 2 plus its weight bytes at 2.5 TB/s.
+// Which instance of a fused kernel to launch: the one that lets two workgroups share a compute unit while the DEC
+// role is not the longer one by a margin (a DEC workgroup that shares its unit takes about 1.2 us longer; the other
+// instance halves the GEMV role's occupancy).  Estimates in microseconds: DEC = its latency floor (launch,
+// activation load, selection, one host-link round trip, merge: about 8) plus the residual bytes at the zero-copy
+// rate of the link (56 GB/s); GEMV = a start-up time plus the packed weight bytes at the rate the format's kernel
+// sustains (fits of the standalone timings at the Llama-3 / Phi-3 shapes).  The ratio at which the choice flips was
+// read off the cost of a launch inside a captured decode step, with either instance forced, cost over the GEMV in
+// us at k_chunk 4 / 6 / 8 / 12 / 16 (shared unit | unit to itself):
+//   any-precision 4096 -> 28672:  1.7 3.3 5.3 9.2 13.3 | 2.6 2.5 3.6 6.9 10.9      flips near DEC = 0.9 GEMV
+//   SqueezeLLM 14336 -> 4096:     2.5 3.4 4.0 6.2 8.4  | 4.2 4.0 3.8 5.6 7.5       near 1.15
+//   SqueezeLLM 4096 -> 28672:     2.4 4.1 6.2 10.0 14.1 | 6.5 6.6 6.8 8.8 9.7      near 1.1
+//   LUT-GEMM 17920 -> 5120:       2.1 2.3 2.6 8.3 12.5 | 6.7 7.5 7.4 8.9 9.7       near 1.25
+//   LUT-GEMM 5120 -> 35840:       1.4 1.9 3.1 3.4 7.2  | 11.0 11.5 12.3 15.5 17.6  beyond 1.27
+enum GemvKind { kAnyprec = 0, kLutgemm = 1, kSqllm = 2 };
+
 double dec_estimate_us(const Config* c) {
     const double k = (double)((uint64_t)c->k_chunk * c->K / 1024u);        // selected rows per call
     return 8.0 + k * (double)c->N * 0.5 / 56e3;
 }
-double gemv_estimate_us(double gemv_bytes) { return 2.0 + gemv_bytes / 2.5e6; }
+double gemv_estimate_us(GemvKind kind, double weight_bytes) {
+    if (kind == kAnyprec) return 2.8 + weight_bytes / 3.7e6;
+    if (kind == kSqllm) return 3.4 + weight_bytes / 4.6e6;
+    return 4.2 + weight_bytes / 3.1e6;
+}
 
-bool fused_two_per_cu(const Config* c, double gemv_bytes) {
+bool fused_two_per_cu(const Config* c, GemvKind kind, double weight_bytes) {
     if (g_opt.fused_two_per_cu >= 0) return g_opt.fused_two_per_cu != 0;
-    return gemv_estimate_us(gemv_bytes) > 1.25 * dec_estimate_us(c);
+    const double flip = kind == kAnyprec ? 0.9 : (kind == kSqllm ? 1.15 : 1.3);
+    return dec_estimate_us(c) < flip * gemv_estimate_us(kind, weight_bytes);
 }
 
 // Whether a fused 3-bit any-precision launch runs both roles in workgroups of `nw` waves (the GEMV's standalone
@@ -797,13 +813,13 @@ bool fused_two_per_cu(const Config* c, double gemv_bytes) {
 // DEC workgroup's host-memory reads hold up the GEMV waves of its compute unit, and the small form spreads the DEC
 // workgroups over four times as many units, so it only pays while the GEMV is the longer role.  Inside a decode step
 // (14336 -> 4096, cost over the GEMV per launch) the small form measured 1.3 / 3.5 / 4.4 / 5.5 / 7.5 us at k_chunk
-// 4 / 8 / 10 / 12 / 16 against 6.6 / 6.4 / 6.4 / 6.4 / 7.1 us: the switch sits where DEC is estimated at 1.4 x the
+// 4 / 8 / 10 / 12 / 16 against 6.6 / 6.4 / 6.4 / 6.4 / 7.1 us: the switch sits where DEC is estimated at 1.7 x the
 // GEMV (k_chunk 14 there).  With 4-wave workgroups (K <= 8192) the 1024-thread form was as fast or faster at every
 // k_chunk.
 bool fused_small(const Config* c, double gemv_bytes, uint32_t nw) {
     if (nw >= 16u || g_opt.fused_small == 0) return false;
     if (g_opt.fused_small > 0) return true;
-    return nw == 8u && dec_estimate_us(c) < 1.4 * gemv_estimate_us(gemv_bytes);
+    return nw == 8u && dec_estimate_us(c) < 1.7 * gemv_estimate_us(kAnyprec, gemv_bytes);
 }
 
 int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
@@ -816,7 +832,7 @@ int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* 
     const bool have_dec = fill_dec_params(c, input, output, true, &dp) == 0;
     const bool fuse = g_opt.fusion && have_dec;
     AnyprecPlan pl;
-    const bool two = fuse && bits == 3 && fused_two_per_cu(c, (double)bits * N * K / 8.0);
+    const bool two = fuse && bits == 3 && fused_two_per_cu(c, kAnyprec, (double)bits * N * K / 8.0);
     hipStream_t s = (hipStream_t)stream;
     if (fuse && bits == 3 && g_opt.fused_small != 0) {
         // Both roles in workgroups of the GEMV's own size (4 or 8 waves): the GEMV keeps its standalone
@@ -867,7 +883,7 @@ int decdec_dec_lutgemm(uint64_t h, const void* input, void* output, const void* 
     if (fuse) {
         LaunchDims d = pl.d;
         d.lds = std::max(d.lds, c->plans[2].lds);
-        d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
+        d.two_per_cu = fused_two_per_cu(c, kLutgemm, (double)bits * N * K / 8.0);
         DD_HIP(launch_dec_lutgemm(dtype, dp, c->plans[2].cg * c->plans[2].sg, pl.p, d, s));
         return kOk;
     }
@@ -890,7 +906,7 @@ int decdec_dec_sqllm(uint64_t h, const void* input, void* output, const void* ma
     if (fuse) {
         LaunchDims d = pl.d;
         d.lds = std::max(d.lds, c->plans[2].lds);
-        d.two_per_cu = fused_two_per_cu(c, (double)bits * N * K / 8.0);
+        d.two_per_cu = fused_two_per_cu(c, kSqllm, (double)bits * N * K / 8.0);
         DD_HIP(launch_dec_sqllm(dtype, dp, c->plans[2].cg * c->plans[2].sg, pl.p, d, s));
         return kOk;
     }
