@@ -79,6 +79,7 @@ def build_layer_set(torch, F, n_layers, k_chunk, seed):
 
 def capture(torch, fn):
     s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())      # the inputs were produced on the current stream
     with torch.cuda.stream(s):
         fn()
     torch.cuda.synchronize()
@@ -116,6 +117,7 @@ def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
     x = torch.randn(1, 1, K, dtype=torch.float16, device="cuda")
     out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
     stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
 
     def launches():
         for i in range(ncopy):
@@ -161,6 +163,7 @@ def kernels_leg(torch, ext, F):
 
     def graph_time(fn, reps=20, iters=20):
         st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(st):
             for _ in range(3):
                 fn()

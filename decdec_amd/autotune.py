@@ -126,6 +126,7 @@ def measure(matrix_dims: dict, algo: str, bitwidth: int, n_tb_values, k_chunk_va
 
     def graph_time(fn):
         st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(st):
             for _ in range(2):
                 fn()

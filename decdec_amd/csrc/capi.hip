@@ -950,6 +950,23 @@ uint64_t decdec_decode_attention_workspace_bytes(uint32_t n_head, uint32_t head_
     return (uint64_t)n_head * nsplit * (head_dim + 2) * 4u;
 }
 
+// Workgroups per query head of the decode attention: as many as the workspace allows, up to 8, without asking for
+// more workgroups than the device has compute units (40 heads x 8 would run in two turns: 6 each).
+static uint32_t attention_splits(uint32_t n_head, uint32_t head_dim, uint64_t workspace_bytes) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    for (uint32_t n = 8; n > 1; --n) {
+        if (n_head * n > (uint32_t)cus && n > 2) continue;
+        if (decdec_decode_attention_workspace_bytes(n_head, head_dim, n) <= workspace_bytes) return n;
+    }
+    return 1;
+}
+
 int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos_device,
                              void* q_out, void* k_cache, void* v_cache, int dtype, uint32_t n_head,
                              uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream) {
@@ -977,9 +994,7 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
     uint32_t nsplit = 1;
     if (workspace != nullptr && max_seq > 256) {
         DD_CHECK(((uintptr_t)workspace % 4) == 0, "workspace must be 4-byte aligned");
-        for (uint32_t n = 8; n > 1; n /= 2) {
-            if (decdec_decode_attention_workspace_bytes(n_head, head_dim, n) <= workspace_bytes) { nsplit = n; break; }
-        }
+        nsplit = attention_splits(n_head, head_dim, workspace_bytes);
     }
     AttentionParams p{q, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
                       1.0f / std::sqrt((float)head_dim), nsplit, (float*)workspace, nullptr, nullptr, nullptr};
@@ -1001,9 +1016,7 @@ int decdec_rope_attention(const void* qkv, const void* cos_table, const void* si
     uint32_t nsplit = 1;
     if (workspace != nullptr && max_seq > 256) {
         DD_CHECK(((uintptr_t)workspace % 4) == 0, "workspace must be 4-byte aligned");
-        for (uint32_t n = 8; n > 1; n /= 2) {
-            if (decdec_decode_attention_workspace_bytes(n_head, head_dim, n) <= workspace_bytes) { nsplit = n; break; }
-        }
+        nsplit = attention_splits(n_head, head_dim, workspace_bytes);
     }
     AttentionParams p{nullptr, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
                       1.0f / std::sqrt((float)head_dim), nsplit, (float*)workspace, qkv, cos_table, sin_table};

@@ -136,12 +136,16 @@ class DecodeStep:
     def capture(self):
         stream = torch.cuda.Stream()
         tok, pos, cnt = self.token.clone(), self.pos.clone(), self.count.clone()
+        # everything queued so far (weights being initialised, the zero fill of the step's own buffers, a prefill)
+        # must have run before the step does: an unordered step would read its token before it was written
+        stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream), torch.no_grad():
             self._step()                      # warm-up: lazy initialisation must not happen under capture
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph, stream=stream), torch.no_grad():
             self._step()
+        torch.cuda.current_stream().wait_stream(stream)
         self.token.copy_(tok); self.pos.copy_(pos); self.count.copy_(cnt)
         torch.cuda.synchronize()
 
