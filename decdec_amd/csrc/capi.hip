@@ -416,21 +416,33 @@ int plan_lutgemm(const void* input, void* output, const void* qw, const void* al
     memset(&p, 0, sizeof(p));
     p.x = input; p.qw = (const uint32_t*)qw; p.alpha = alpha; p.q_bias = q_bias; p.out = output;
     p.N = N; p.K = K; p.bits = (uint32_t)bits; p.group_size = (uint32_t)group_size;
-    // 16 waves per workgroup share 64 columns and split the workgroup's K range in slices of 1..4 tiles
-    // (tables of 4 tiles per wave = 32 KB of LDS); enough K ranges for about 8 waves per SIMD
+    // 16 waves per workgroup share 64 columns and split the workgroup's K range in slices of 1..7 tiles of 32
+    // channels per wave (tables of 7 tiles per wave = 57 KB of LDS; two workgroups fit a compute unit).  The number
+    // of K ranges (one atomic add, i.e. one rounding of a 16-bit output, each; at most 9) is the one with the
+    // smallest (turns of workgroups) x (tiles per wave + start-up): a grid a little above one turn runs its rest as
+    // a second, nearly empty turn.  Measured: 5120 -> 7680 with 600 workgroups 8.8 us, with 480 7.7 us;
+    // 17920 -> 5120 with 720 workgroups 14.2 us, with 400 (7 tiles per wave) 12.6 us; 5120 -> 35840 with 1680
+    // workgroups 26.5 us, with 1120 25.1 us.
     const uint32_t waves = 16, tiles = K / 32;
     p.n_tiles = cdiv(N, 64);
-    uint32_t kt = g_opt.lutgemm_ktiles > 0 ? (uint32_t)g_opt.lutgemm_ktiles : cdiv(8192, p.n_tiles * waves);
-    kt = std::max(1u, kt);
-    p.slice_tiles = std::max(1u, std::min(4u, cdiv(tiles, kt * waves)));
-    p.k_tiles = cdiv(tiles, p.slice_tiles * waves);
-    // Two 16-wave workgroups fit a compute unit; a grid a little above that many workgroups runs its rest as a
-    // second, nearly empty turn (5120 -> 7680: 600 workgroups 8.8 us, 480 workgroups 7.8 us): fewer K ranges then.
-    const uint32_t slots = 2u * device_cus();
-    while (g_opt.lutgemm_ktiles <= 0 && kt > 1 && p.n_tiles * p.k_tiles > slots && p.n_tiles * p.k_tiles < 2u * slots) {
-        --kt;
+    if (g_opt.lutgemm_ktiles > 0) {
+        const uint32_t kt = (uint32_t)g_opt.lutgemm_ktiles;
         p.slice_tiles = std::max(1u, std::min(4u, cdiv(tiles, kt * waves)));
         p.k_tiles = cdiv(tiles, p.slice_tiles * waves);
+    } else {
+        const uint32_t slots = 2u * device_cus();
+        uint32_t best_cost = ~0u;
+        for (uint32_t kr = 1; kr <= 9; ++kr) {
+            const uint32_t slice = cdiv(tiles, kr * waves);
+            if (slice > 7u) continue;
+            const uint32_t k_tiles = cdiv(tiles, slice * waves);
+            const uint32_t cost = cdiv(p.n_tiles * k_tiles, slots) * (2u * slice + 3u);
+            if (cost < best_cost) { best_cost = cost; p.slice_tiles = slice; p.k_tiles = k_tiles; }
+        }
+        if (best_cost == ~0u) {                          // K beyond 9 ranges of 7 tiles per wave: more ranges
+            p.slice_tiles = 7u;
+            p.k_tiles = cdiv(tiles, p.slice_tiles * waves);
+        }
     }
     pl->d.grid = p.n_tiles * p.k_tiles;
     pl->d.block = 64u * waves;
