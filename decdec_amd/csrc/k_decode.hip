@@ -60,9 +60,10 @@ __device__ __forceinline__ float group_sum(float v) {
 // D/8 lanes owns a cache position (16 bytes of K and of V per lane); a wave visits 64 / (D/8) positions per step
 // and four steps per loop trip (their rows requested together), the 16 waves interleave, every lane group keeps
 // its own running maximum / sum / output (online softmax), and the groups are merged through LDS.  With
-// nsplit > 1 every workgroup leaves (max, sum, output) of its range in the workspace and a second, small kernel
-// merges the ranges of a head (a merge by the workgroup that finishes last would need device-scope fences, which
-// write back and invalidate whole L2 caches on this multi-die GPU: measured 110 us per launch).
+// nsplit > 1 every workgroup leaves (max, sum, output) of its range in the workspace and the ranges of a head are
+// merged either by the workgroup of the head that arrives last (see the end of the kernel) or by a second, small
+// kernel (a merge behind device-scope fences writes back and invalidates whole L2 caches on this multi-die GPU:
+// measured 110 us per launch).
 template <int DT, int D>
 __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionParams p) {
     using E = Elem<DT>;
@@ -202,12 +203,58 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
         if (tid < (uint32_t)D) E::store(p.out, (size_t)h * D + tid, O / L);
         return;
     }
-    // partial result of this range: [D] outputs, then the maximum and the sum; a second kernel merges them
+    // partial result of this range: [D] outputs, then the maximum and the sum
     float* ws = p.workspace + ((size_t)h * nsplit + split) * (D + 2);
-    if (tid < (uint32_t)D) {
-        ws[tid] = O;
-        if (tid == 0) { ws[D] = M; ws[D + 1] = L; }
+    if (p.counters == nullptr) {                     // a second kernel merges the ranges
+        if (tid < (uint32_t)D) {
+            ws[tid] = O;
+            if (tid == 0) { ws[D] = M; ws[D + 1] = L; }
+        }
+        return;
     }
+    // Merge by the workgroup of the head that finishes last, without fences (a device-scope fence writes back and
+    // invalidates a whole L2 on this multi-die GPU): the partial results travel as relaxed device-scope atomic
+    // stores and loads, which go past the L2 to memory; a workgroup counts itself in only after its stores have been
+    // acknowledged, so whoever draws the last number finds every range's result in memory.
+    if (tid < (uint32_t)D) {
+        __hip_atomic_store(ws + tid, O, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            __hip_atomic_store(ws + D, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(ws + D + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    uint32_t* flag = (uint32_t*)pm;                  // the maxima are no longer read
+    if (tid == 0) {
+        const uint32_t drawn = __hip_atomic_fetch_add(p.counters + h, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        flag[0] = (drawn + 1u == nsplit) ? 1u : 0u;
+        if (drawn + 1u == nsplit) __hip_atomic_store(p.counters + h, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+    }
+    __syncthreads();
+    if (flag[0] == 0u || tid >= (uint32_t)D) return;
+    const float* wh = p.workspace + (size_t)h * nsplit * (D + 2);
+    float ms[8], ls[8], os[8];
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) {
+        const uint32_t c = (uint32_t)sp < nsplit ? (uint32_t)sp : 0u;          // all loads in flight together
+        ms[sp] = __hip_atomic_load(wh + (size_t)c * (D + 2) + D, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ls[sp] = __hip_atomic_load(wh + (size_t)c * (D + 2) + D + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        os[sp] = __hip_atomic_load(wh + (size_t)c * (D + 2) + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    float Mg = -__builtin_inff();
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) if ((uint32_t)sp < nsplit && ms[sp] > Mg) Mg = ms[sp];
+    float Lg = 0.f, Og = 0.f;
+#pragma unroll
+    for (int sp = 0; sp < 8; ++sp) {
+        if ((uint32_t)sp < nsplit) {
+            const float w = (ms[sp] == -__builtin_inff()) ? 0.f : __expf(ms[sp] - Mg);
+            Lg += ls[sp] * w;
+            Og += os[sp] * w;
+        }
+    }
+    E::store(p.out, (size_t)h * D + tid, Og / Lg);
 }
 
 // Second step with nsplit > 1: one workgroup of D threads per head combines the ranges' partial results.
@@ -419,7 +466,7 @@ size_t decode_attention_lds_bytes(uint32_t head_dim) {
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s) {
     const dim3 grid(p.n_head * p.nsplit), block(1024), mgrid(p.n_head);
     const size_t lds = decode_attention_lds_bytes(p.head_dim);
-    const bool merge = p.nsplit > 1;
+    const bool merge = p.nsplit > 1 && p.counters == nullptr;
     if (dt == kFP16 && p.head_dim == 128) {
         hipLaunchKernelGGL((decode_attention_kernel<kFP16, 128>), grid, block, lds, s, p);
         if (merge) hipLaunchKernelGGL((decode_attention_merge_kernel<kFP16, 128>), mgrid, dim3(128), 0, s, p);

@@ -70,6 +70,9 @@ struct AttentionParams {
     const void* qkv;                 // [(n_head + 2 n_kv) * head_dim]
     const void* cos_table;           // [max_seq][head_dim]
     const void* sin_table;
+    // [n_head] arrival counters behind the partial results in the workspace, zero between calls (null: the ranges are
+    // merged by a second kernel)
+    uint32_t* counters;
 };
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);

@@ -29,7 +29,9 @@ def rope_cache_update(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: tor
 
 
 def attention_workspace(n_head: int, head_dim: int, device="cuda") -> torch.Tensor:
-    """Workspace that lets `decode_attention` share the positions of a head among 8 workgroups."""
+    """Workspace that lets `decode_attention` / `rope_attention` share the positions of a head among up to 8
+    workgroups.  It must be zero when first used (it starts with the heads' arrival counters, which every call leaves
+    at zero)."""
     n = _lib.load().decdec_decode_attention_workspace_bytes(n_head, head_dim, 8)
     return torch.zeros(n // 4, dtype=torch.float32, device=device)
 

@@ -60,6 +60,7 @@ int decdec_version(void);
  * "fused_small" (fused 3-bit any-precision launches with both roles in the GEMV's own 4- or 8-wave workgroups:
  * -1 = when those have 5 to 8 waves [default], 1 = whenever they have at most 8, 0 = never), "anyprec_rg" (row
  * groups per any-precision workgroup, 0 = automatic),
+ * "attention_two_step" (decode attention with a workspace: 1 = merge in a second kernel, 0 = in the kernel [default]),
  * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
@@ -158,9 +159,11 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     ([n_kv_head][max_seq][head_dim]).  A position outside [0, max_seq) writes nothing.
  *   decdec_decode_attention: out[h] = softmax(q[h] . K[kv(h)][0..pos] / sqrt(head_dim)) V[kv(h)][0..pos],
  *     head_dim 64 or 128, grouped-query heads (kv(h) = h / (n_head / n_kv_head)).  With a workspace of
- *     decdec_decode_attention_workspace_bytes(n_head, head_dim, 8) bytes (caller-owned device memory, contents
- *     irrelevant; one workspace serves any number of calls that do not overlap in time) the positions of a head
- *     are shared by 8 workgroups and a second small kernel merges them; workspace NULL = one workgroup per head.
+ *     decdec_decode_attention_workspace_bytes(n_head, head_dim, 8) bytes (caller-owned device memory, ZERO when
+ *     first used: it starts with one arrival counter per head, which every call leaves at zero; one workspace serves
+ *     any number of calls that do not overlap in time) the positions of a head are shared by up to 8 workgroups (no
+ *     more workgroups than the device has compute units) and the workgroup of a head that finishes last merges
+ *     them (option "attention_two_step" = 1: a second small kernel does); workspace NULL = one workgroup per head.
  *   decdec_rope_attention: the two calls above in one launch (plus the merge kernel when a workspace is given): takes
  *     the un-rotated qkv, rotates the queries and the new key on the fly (rounded to the storage type; a value
  *     within rounding error of a tie may differ by one unit in the last place from what decdec_rope_cache_update

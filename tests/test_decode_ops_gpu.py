@@ -119,6 +119,32 @@ def test_rope_attention_equals_the_two_step_form(H, Hkv, hd, S, dt):
     assert torch.equal(kc, k0) and torch.equal(vc, v0) and torch.isfinite(out.float()).all()
 
 
+@pytest.mark.parametrize("H,Hkv,hd,S", [(32, 8, 128, 2048), (40, 10, 128, 1100)])
+def test_attention_ranges_merged_in_kernel_over_many_calls(H, Hkv, hd, S):
+    """The workgroup of a head that finishes last merges the head's ranges from results the others left in the
+    workspace (no second kernel, no fence): several hundred calls in a row at random positions against the
+    one-workgroup-per-head form, then the two-step form on the same workspace; the counters end at zero."""
+    from decdec_amd import _lib
+    g = torch.Generator(device="cuda").manual_seed(7)
+    kc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").half()
+    vc = torch.randn(1, Hkv, S, hd, generator=g, device="cuda").half()
+    ws = D.attention_workspace(H, hd)
+    one, many = (torch.empty(H * hd, dtype=torch.float16, device="cuda") for _ in range(2))
+    positions = torch.randint(0, S, (400,), generator=g, device="cuda").tolist()
+    try:
+        for i, pos in enumerate(positions):
+            if i == 300:
+                _lib.set_option("attention_two_step", 1)
+            q = (torch.randn(H * hd, generator=g, device="cuda") * 1.5).half()
+            p = torch.tensor([pos], device="cuda")
+            D.decode_attention(q, kc, vc, p, one, H, Hkv)
+            D.decode_attention(q, kc, vc, p, many, H, Hkv, ws)
+            assert _close(many, one, 3e-3), (i, pos)
+    finally:
+        _lib.set_option("attention_two_step", 0)
+    assert int(ws.view(torch.int32)[:H].abs().sum()) == 0
+
+
 @pytest.mark.parametrize("n", [1, 255, 14336])
 def test_silu_mul(n):
     gu = torch.randn(2 * n, device="cuda").half() * 3
