@@ -53,6 +53,7 @@ SIGNATURES = {
     "decdec_rope_cache_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp],
     "decdec_decode_attention": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp, _u64, _vp],
     "decdec_rope_attention": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp, _u64, _vp],
+    "decdec_dense_gemv": [_vp, _vp, _vp, _i32, _u32, _u32, _vp],
     "decdec_silu_mul": [_vp, _vp, _i32, _u32, _vp],
     "decdec_add_rmsnorm": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp],
     "decdec_greedy_pick": [_vp, _u32, _i32, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp],

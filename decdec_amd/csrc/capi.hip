@@ -1058,6 +1058,16 @@ int decdec_rope_attention(const void* qkv, const void* cos_table, const void* si
     return kOk;
 }
 
+int decdec_dense_gemv(const void* weight, const void* x, void* out, int dtype, uint32_t N, uint32_t K, void* stream) {
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    DD_CHECK(weight && x && out, "null pointer argument");
+    DD_CHECK(K >= 8 && K % 8 == 0, "in_features must be a positive multiple of 8, got %u", K);
+    DD_CHECK(((uintptr_t)weight % 16) == 0 && ((uintptr_t)x % 16) == 0, "weight and x must be 16-byte aligned");
+    if (N == 0) return kOk;
+    DD_HIP(launch_dense_gemv(dtype, weight, x, out, N, K, (hipStream_t)stream));
+    return kOk;
+}
+
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream) {
     DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
     DD_CHECK(gate_up && out, "null pointer argument");

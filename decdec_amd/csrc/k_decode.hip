@@ -295,6 +295,83 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ 
     E::store(out, i, a / (1.f + __expf(-a)) * b);
 }
 
+// ---- dense 16-bit GEMV: the unquantised output head of a decoder ------------------------------------------
+// out[n] = sum_k W[n][k] x[k], W row-major.  Bound by the read of W (the head of an 8B model is a gigabyte per
+// token), so the kernel is a stream: a wave owns four rows, a lane 16 bytes of each per step of 512 columns, two
+// steps (eight 16-byte loads of W per lane, never reused, hence non-temporal) in flight together; x comes through
+// the vector cache (every wave reads the same few KB).  Products accumulate in fp32, one rounding at the store.
+typedef uint32_t u32x4_nt __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ float dot8(const u32x4& w, const u32x4& x, float acc) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if constexpr (DT == kFP16) {
+            half2_t a, b;
+            const uint32_t wa = w[j], xb = x[j];
+            __builtin_memcpy(&a, &wa, 4); __builtin_memcpy(&b, &xb, 4);
+            acc = __builtin_amdgcn_fdot2(a, b, acc, false);
+        } else {
+            acc = __builtin_fmaf(__uint_as_float(w[j] << 16), __uint_as_float(x[j] << 16), acc);
+            acc = __builtin_fmaf(__uint_as_float(w[j] & 0xFFFF0000u), __uint_as_float(x[j] & 0xFFFF0000u), acc);
+        }
+    }
+    return acc;
+}
+
+constexpr int kDenseRows = 4;          // rows per wave
+constexpr int kDenseWaves = 4;         // waves per workgroup
+
+template <int DT>
+__global__ __launch_bounds__(kDenseWaves * 64) void dense_gemv_kernel(const void* __restrict__ weight,
+                                                                      const void* __restrict__ x, void* __restrict__ out,
+                                                                      const uint32_t N, const uint32_t K) {
+    using E = Elem<DT>;
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t row0 = (blockIdx.x * (uint32_t)kDenseWaves + wave) * (uint32_t)kDenseRows;
+    if (row0 >= N) return;
+    const uint16_t* wr[kDenseRows];
+#pragma unroll
+    for (int r = 0; r < kDenseRows; ++r) {
+        const uint32_t rr = row0 + r < N ? row0 + r : N - 1u;      // rows past the end re-read the last one; not stored
+        wr[r] = (const uint16_t*)weight + (size_t)rr * K;
+    }
+    float acc[kDenseRows] = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t steps = (K + 511u) / 512u;
+    for (uint32_t s = 0; s < steps; s += 2u) {
+        u32x4 wv[2][kDenseRows], xv[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const uint32_t col = ((s + u) * 64u + lane) * 8u;
+            const bool ok = col < K;                               // K is a multiple of 8
+            const uint32_t c = ok ? col : 0u;
+            xv[u] = *(const u32x4*)((const uint16_t*)x + c);
+            if (!ok) xv[u] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int r = 0; r < kDenseRows; ++r) wv[u][r] = __builtin_nontemporal_load((const u32x4*)(wr[r] + c));
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < kDenseRows; ++r) acc[r] = dot8<DT>(wv[u][r], xv[u], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kDenseRows; ++r) acc[r] = wave_sum(acc[r]);
+    if (lane < (uint32_t)kDenseRows && row0 + lane < N) {
+        const float v = lane == 0 ? acc[0] : (lane == 1 ? acc[1] : (lane == 2 ? acc[2] : acc[3]));
+        E::store(out, row0 + lane, v);
+    }
+}
+
+hipError_t launch_dense_gemv(int dt, const void* weight, const void* x, void* out, uint32_t N, uint32_t K, hipStream_t s) {
+    const uint32_t rows_per_block = (uint32_t)(kDenseRows * kDenseWaves);
+    const dim3 grid((N + rows_per_block - 1u) / rows_per_block), block(kDenseWaves * 64);
+    if (dt == kFP16) hipLaunchKernelGGL((dense_gemv_kernel<kFP16>), grid, block, 0, s, weight, x, out, N, K);
+    else if (dt == kBF16) hipLaunchKernelGGL((dense_gemv_kernel<kBF16>), grid, block, 0, s, weight, x, out, N, K);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 // h = x + y (skipped when y is null), normed = h / rms(h) * weight: the residual add and the RMS normalisation that
 // follows it in a decoder block.  One workgroup per row, four neighbouring elements per thread and pass (one 8-byte
 // load each of x, y and the weight, all requested before anything is used), statistics in fp32.

@@ -76,6 +76,7 @@ struct AttentionParams {
 };
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);
+hipError_t launch_dense_gemv(int dt, const void* weight, const void* x, void* out, uint32_t N, uint32_t K, hipStream_t s);
 hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, hipStream_t s);
 size_t greedy_pick_workspace_bytes();
 hipError_t launch_greedy_pick(int dt, const void* logits, uint32_t n, void* workspace, float* copy_out, long long* token,

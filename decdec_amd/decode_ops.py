@@ -70,6 +70,15 @@ def rope_attention(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.
                                                  workspace.numel() * 4 if workspace is not None else 0, _stream()))
 
 
+def dense_gemv(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n] = sum_k weight[n, k] * x[k] for an unquantised fp16 / bf16 weight [N, K] (overwrites out)."""
+    _half_cuda(weight, x, out)
+    _check(weight.dim() == 2 and x.numel() == weight.shape[1] and out.numel() == weight.shape[0],
+           "weight [N, K], x with K and out with N elements")
+    _lib.check(_lib.load().decdec_dense_gemv(_ptr(weight), _ptr(x), _ptr(out), _dt(out), weight.shape[0],
+                                             weight.shape[1], _stream()))
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _half_cuda(gate_up, out)
     _check(gate_up.numel() == 2 * out.numel(), "gate_up must hold twice as many elements as out")

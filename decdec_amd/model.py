@@ -272,6 +272,11 @@ class Transformer(nn.Module):
                 h, branch = layer.decode_step(h, branch, input_pos, full)
             n = torch.empty_like(h)
             decode_ops.add_rmsnorm(h, branch, self.norm.weight, torch.empty_like(h), n, self.norm.eps)
+            if self.output.bias is None and self.output.weight.dtype == n.dtype and self.config.dim % 8 == 0:
+                # the unquantised head on the library's streaming GEMV (a gigabyte of weights per token at 8B)
+                logits = torch.empty(1, 1, self.config.vocab_size, dtype=n.dtype, device=n.device)
+                decode_ops.dense_gemv(self.output.weight, n.view(-1), logits.view(-1))
+                return logits
             return self.output(n)
         mask = self.causal_mask.index_select(0, input_pos)                     # [S, max_seq]
         cos, sin = self.rope_cos.index_select(0, input_pos), self.rope_sin.index_select(0, input_pos)

@@ -170,6 +170,9 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  *     stores), attends cache rows 0 .. pos - 1 and the new row, and appends the new
  *     key / value row to the caches (position outside [0, max_seq): nothing is appended, rows 0 .. max_seq - 1 are
  *     attended).  qkv, the tables and the caches 16-byte aligned.
+ *   decdec_dense_gemv: out[n] = sum_k weight[n][k] * x[k] for an unquantised row-major fp16 / bf16 weight [N][K]
+ *     (a decoder's output head), fp32 accumulation, `out` is overwritten (not accumulated).  K a multiple of 8,
+ *     weight and x 16-byte aligned.
  *   decdec_silu_mul: out[i] = silu(gate_up[i]) * gate_up[n + i], i < n.
  *   decdec_add_rmsnorm: per row of `dim` elements (a multiple of 4, <= 16384; 8-byte aligned tensors), h = x + y rounded to the storage type and written to
  *     h_out (y and h_out may be NULL: then h = x), normed_out = h / sqrt(mean(h^2) + eps) * weight.
@@ -192,6 +195,8 @@ int decdec_rope_attention(const void* qkv, const void* cos_table, const void* si
                           const int64_t* pos_device, void* out, void* k_cache, void* v_cache, int dtype,
                           uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq,
                           void* workspace, uint64_t workspace_bytes, void* stream);
+int decdec_dense_gemv(const void* weight, const void* x, void* out, int dtype, uint32_t N, uint32_t K,
+                      void* stream);
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
 int decdec_add_rmsnorm(const void* x, const void* y, const void* weight, void* h_out, void* normed_out,
                        int dtype, uint32_t rows, uint32_t dim, float eps, void* stream);

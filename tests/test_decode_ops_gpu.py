@@ -145,6 +145,21 @@ def test_attention_ranges_merged_in_kernel_over_many_calls(H, Hkv, hd, S):
     assert int(ws.view(torch.int32)[:H].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,K", [(640, 512), (1001, 4096), (32064, 5120), (7, 8), (130, 1032), (4099, 8192)])
+def test_dense_gemv(N, K, dt):
+    g = torch.Generator().manual_seed(N + K)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dt).cuda()
+    x = torch.randn(K, generator=g).to(dt).cuda()
+    out = torch.full((N,), 3.0, dtype=dt, device="cuda")
+    D.dense_gemv(w, x, out)
+    want = w.double() @ x.double()
+    # one rounding of an fp32 sum: half a unit in the last place of the result plus the fp32 accumulation error
+    ulp = 2.0 ** (-11 if dt == torch.float16 else -8)
+    tol = ulp * want.abs() + 1e-5 * (w.double().abs() @ x.double().abs())
+    assert bool(((out.double() - want).abs() <= 1.001 * tol).all()), float(((out.double() - want).abs() / tol).max())
+
+
 @pytest.mark.parametrize("n", [1, 255, 14336])
 def test_silu_mul(n):
     gu = torch.randn(2 * n, device="cuda").half() * 3
