@@ -389,9 +389,11 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     // dword-aligned activation vector (it is read through the scalar cache)
     const bool tile_able = bits == 3 && K % 1024 == 0 && ((uintptr_t)qweight % 16) == 0 &&
                            ((uintptr_t)input % 4) == 0 && g_opt.anyprec_tile != 0;
-    if (tile_able) {
-        uint32_t cs = (g_opt.anyprec_tile == 2 || g_opt.anyprec_tile == 4) ? (uint32_t)g_opt.anyprec_tile : 8u;
-        while (cs < 8u && p.W / (4u * cs) > 16u) cs *= 2u;   // at most 16 atomic adds (roundings) per 16-bit output
+    // at most 8 atomic adds (roundings, in an order that varies from run to run) per 16-bit output: with 14 of them
+    // (K = 14336) an output now and then missed the 1e-2 bound by a few percent of it; longer rows keep the row form
+    uint32_t cs = (g_opt.anyprec_tile == 2 || g_opt.anyprec_tile == 4) ? (uint32_t)g_opt.anyprec_tile : 8u;
+    while (cs < 8u && p.W / (4u * cs) > 8u) cs *= 2u;
+    if (tile_able && p.W / (4u * cs) <= 8u) {
         p.tile_cs = cs;
         p.tile_kt = p.W / (4u * cs);
         p.tiles = cdiv(N, 64) * p.tile_kt;

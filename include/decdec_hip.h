@@ -54,7 +54,7 @@ int decdec_version(void);
 
 /* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
  * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
- * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "anyprec_tile" (3-bit LDS-transposed tile decoder, waves per tile 2/4/8, 0 = off [default]), "lutgemm_ktiles",
+ * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "anyprec_tile" (3-bit LDS-transposed tile decoder for K <= 8192, waves per tile 2/4/8, 0 = off [default]), "lutgemm_ktiles",
  * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "fused_two_per_cu" (fused launches: 1 / 0 = always /
  * never the kernel instance that lets two workgroups share a compute unit, -1 = chosen per launch [default]),
  * "fused_small" (fused 3-bit any-precision launches with both roles in the GEMV's own 4- or 8-wave workgroups:
