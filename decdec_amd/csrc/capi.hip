@@ -57,6 +57,7 @@ struct Options {
     int dec_block_waves = 16;   // waves of a standalone DEC workgroup: 4, 8 or 16
     int fused_two_per_cu = -1;  // fused launches: 1 / 0 = always / never two workgroups per compute unit, -1 = by estimate
     int attention_two_step = 0; // decode attention with a workspace: 1 = merge the ranges of a head in a second kernel
+    int attention_single_below = 512;  // ... and merging in the kernel: sequences up to this length are not shared at all
     int fused_small = -1;       // fused 3-bit any-precision launches with both roles in the GEMV's own smaller workgroups:
                                 // -1 = when those have 5..8 waves (measured faster there), 1 = whenever they have <= 8, 0 = never
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
@@ -84,6 +85,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "fused_two_per_cu")) return &g_opt.fused_two_per_cu;
     if (!strcmp(name, "fused_small")) return &g_opt.fused_small;
     if (!strcmp(name, "attention_two_step")) return &g_opt.attention_two_step;
+    if (!strcmp(name, "attention_single_below")) return &g_opt.attention_single_below;
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     return nullptr;
 }
@@ -1031,7 +1033,8 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
     AttentionParams p{q, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
                       1.0f / std::sqrt((float)head_dim), nsplit, nsplit > 1 ? (float*)workspace + n_head : nullptr,
                       nullptr, nullptr, nullptr,
-                      (nsplit > 1 && g_opt.attention_two_step == 0) ? (uint32_t*)workspace : nullptr};
+                      (nsplit > 1 && g_opt.attention_two_step == 0) ? (uint32_t*)workspace : nullptr,
+                      (uint32_t)std::max(0, g_opt.attention_single_below)};
     DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
     return kOk;
 }
@@ -1055,7 +1058,8 @@ int decdec_rope_attention(const void* qkv, const void* cos_table, const void* si
     AttentionParams p{nullptr, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
                       1.0f / std::sqrt((float)head_dim), nsplit, nsplit > 1 ? (float*)workspace + n_head : nullptr,
                       qkv, cos_table, sin_table,
-                      (nsplit > 1 && g_opt.attention_two_step == 0) ? (uint32_t*)workspace : nullptr};
+                      (nsplit > 1 && g_opt.attention_two_step == 0) ? (uint32_t*)workspace : nullptr,
+                      (uint32_t)std::max(0, g_opt.attention_single_below)};
     DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
     return kOk;
 }

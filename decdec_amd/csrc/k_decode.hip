@@ -75,11 +75,16 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
     float* po = pl + NG;                    // [NG][D] outputs
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t sub = lane / LPP, dl = lane % LPP;
-    const uint32_t nsplit = p.nsplit, h = blockIdx.x / nsplit, split = blockIdx.x % nsplit;
+    const uint32_t h = blockIdx.x / p.nsplit, split = blockIdx.x % p.nsplit;
     const uint32_t kvh = h / (p.n_head / p.n_kv);
     const uint16_t* kc = (const uint16_t*)p.k_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
     const uint16_t* vc = (const uint16_t*)p.v_cache + (size_t)kvh * p.max_seq * D + 8 * dl;
     long long pos64 = *p.pos;
+    // Short sequences: sharing a head's positions between workgroups costs more (partial results, a counter, a
+    // second pass: about 3 us of memory round trips) than it saves, so the head's first workgroup takes them all.
+    const bool alone = p.counters != nullptr && pos64 + 1 <= (long long)p.single_below;
+    if (alone && split != 0u) return;
+    const uint32_t nsplit = alone ? 1u : p.nsplit;
     const bool fused = p.qkv != nullptr;
     const bool in_cache = pos64 >= 0 && pos64 < (long long)p.max_seq;      // the new token has a cache row
     if (pos64 < 0) pos64 = 0;
@@ -136,6 +141,10 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
     float m = -__builtin_inff(), l = 0.f, o[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = 0.f;
+    // The scan is bound by the instruction issue of the workgroup's compute unit, so it is written to need few
+    // instructions: fp16 scores come from packed dot products of the raw registers (fp32 accumulation, scaled
+    // afterwards), and the UN rows of a trip share one update of the running maximum (one rescaling of the output
+    // instead of UN).
     for (uint32_t p0 = lo + wave * PPW; p0 < hi; p0 += UN * 16 * PPW) {
         u32x4 kr[UN], vr[UN];
 #pragma unroll
@@ -146,26 +155,55 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
             vr[u] = *(const u32x4*)(vc + (size_t)ppc * D);
             if (ppc == newpos) { kr[u] = knew; vr[u] = vnew; }             // the new token's row is not in the cache yet
         }
+        float sc[UN];
+        float mn = m;
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const bool valid = p0 + (uint32_t)u * 16 * PPW + sub < hi;
-            float s = 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                s += q[2 * e] * E::from_raw(kr[u][e] & 0xFFFFu);
-                s += q[2 * e + 1] * E::from_raw(kr[u][e] >> 16);
-            }
-            s = group_sum<LPP>(s);
-            if (valid) {
-                const float mn = s > m ? s : m;
-                const float corr = __expf(m - mn), pr = __expf(s - mn);        // m = -inf: corr = 0
-                l = l * corr + pr;
+            float t = 0.f;
+            if constexpr (DT == kFP16) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    o[2 * e] = o[2 * e] * corr + pr * E::from_raw(vr[u][e] & 0xFFFFu);
-                    o[2 * e + 1] = o[2 * e + 1] * corr + pr * E::from_raw(vr[u][e] >> 16);
+                    half2_t a, b;
+                    const uint32_t ka = kr[u][e], qb = qr[e];
+                    __builtin_memcpy(&a, &ka, 4); __builtin_memcpy(&b, &qb, 4);
+                    t = __builtin_amdgcn_fdot2(a, b, t, false);
                 }
-                m = mn;
+                t = group_sum<LPP>(t) * p.scale;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    t += q[2 * e] * E::from_raw(kr[u][e] & 0xFFFFu);
+                    t += q[2 * e + 1] * E::from_raw(kr[u][e] >> 16);
+                }
+                t = group_sum<LPP>(t);
+            }
+            const bool valid = p0 + (uint32_t)u * 16 * PPW + sub < hi;
+            sc[u] = valid ? t : -__builtin_inff();
+            mn = sc[u] > mn ? sc[u] : mn;
+        }
+        // a lane group without a row in the trip (mn still -inf) changes nothing: its weights are exp(-inf - 0) = 0
+        const float mb = mn == -__builtin_inff() ? 0.f : mn;
+        const float corr = mn == -__builtin_inff() ? 1.f : __expf(m - mn); // m = -inf, mn finite: corr = 0
+        m = mn;
+        l *= corr;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] *= corr;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const float pr = __expf(sc[u] - mb);                           // a row past the range: exp(-inf) = 0
+            l += pr;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if constexpr (DT == kFP16) {
+                    half2_t v2;
+                    const uint32_t vv = vr[u][e];
+                    __builtin_memcpy(&v2, &vv, 4);
+                    o[2 * e] = __builtin_fmaf(pr, (float)v2[0], o[2 * e]);
+                    o[2 * e + 1] = __builtin_fmaf(pr, (float)v2[1], o[2 * e + 1]);
+                } else {
+                    o[2 * e] = __builtin_fmaf(pr, E::from_raw(vr[u][e] & 0xFFFFu), o[2 * e]);
+                    o[2 * e + 1] = __builtin_fmaf(pr, E::from_raw(vr[u][e] >> 16), o[2 * e + 1]);
+                }
             }
         }
     }

@@ -73,6 +73,9 @@ struct AttentionParams {
     // [n_head] arrival counters behind the partial results in the workspace, zero between calls (null: the ranges are
     // merged by a second kernel)
     uint32_t* counters;
+    // with counters: a sequence of at most this many positions is scanned by the first workgroup of a head alone
+    // (no partial results, no merge; the other workgroups of the head return at once)
+    uint32_t single_below;
 };
 hipError_t launch_rope_cache(int dt, const RopeCacheParams& p, hipStream_t s);
 hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t s);

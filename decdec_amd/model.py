@@ -236,9 +236,10 @@ class Transformer(nn.Module):
         cos, sin = rope_tables(self.config.head_dim, max_seq_length, self.config.rope_base, dev)
         self.rope_cos, self.rope_sin = cos.to(self.dtype), sin.to(self.dtype)
         self.attention_workspace = None
-        # caches beyond 1024 positions: a head's positions are shared by 8 workgroups (slower by a microsecond below
-        # ~900 positions, 9.6 against 17.9 us at 2047)
-        if self.decode_kernels and max_seq_length > 1024:
+        # caches beyond 512 positions: with a workspace the kernel shares a head's positions among up to 8 workgroups
+        # once the sequence is longer than that (8.9 against 17.0 us at position 2047; below, one workgroup per head
+        # is faster: 5.9 against 8.0 us at 255)
+        if self.decode_kernels and max_seq_length > 512:
             from . import decode_ops
             self.attention_workspace = decode_ops.attention_workspace(self.config.n_head, self.config.head_dim, dev)
 

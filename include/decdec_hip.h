@@ -61,6 +61,8 @@ int decdec_version(void);
  * -1 = when those have 5 to 8 waves [default], 1 = whenever they have at most 8, 0 = never), "anyprec_rg" (row
  * groups per any-precision workgroup, 0 = automatic),
  * "attention_two_step" (decode attention with a workspace: 1 = merge in a second kernel, 0 = in the kernel [default]),
+ * "attention_single_below" (... merging in the kernel: sequences of at most this many positions are scanned by one
+ * workgroup per head, which is faster there; default 512, 0 = always share),
  * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);

@@ -5,7 +5,7 @@ import math
 import pytest
 import torch
 
-from decdec_amd import decode_ops as D, generate as G
+from decdec_amd import _lib, decode_ops as D, generate as G
 from decdec_amd.model import apply_rope, rope_tables
 
 pytestmark = pytest.mark.gpu
@@ -57,14 +57,22 @@ def test_decode_attention(H, Hkv, hd, S, dt):
         q = (torch.randn(H * hd, generator=g, device="cuda") * 1.5).to(dt)
         out = torch.empty(H * hd, dtype=dt, device="cuda")
         D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out, H, Hkv)
-        out_s = torch.empty(H * hd, dtype=dt, device="cuda")        # positions shared by 8 workgroups per head
-        D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out_s, H, Hkv, ws)
+        # with a workspace: positions shared by up to 8 workgroups per head, short sequences (<= 512 positions by
+        # default) scanned by the head's first workgroup alone; with the option at 0 every length is shared
+        out_s, out_a = (torch.empty(H * hd, dtype=dt, device="cuda") for _ in range(2))
+        D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out_a, H, Hkv, ws)
+        _lib.set_option("attention_single_below", 0)
+        try:
+            D.decode_attention(q, kc, vc, torch.tensor([pos], device="cuda"), out_s, H, Hkv, ws)
+        finally:
+            _lib.set_option("attention_single_below", 512)
         k = kc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)       # [H, L, hd]
         v = vc[0, :, :pos + 1].float().repeat_interleave(H // Hkv, dim=0)
         att = torch.softmax(torch.einsum("hd,hld->hl", q.float().view(H, hd), k) / math.sqrt(hd), dim=-1)
         want = torch.einsum("hl,hld->hd", att, v)
         assert _close(out.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos,)
         assert _close(out_s.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos, "split")
+        assert _close(out_a.view(H, hd), want, 2e-2 if dt == torch.bfloat16 else 3e-3), (pos, "split or alone")
     # a position beyond the cache attends the whole cache and reads nothing outside it
     D.decode_attention(q, kc, vc, torch.tensor([S + 100], device="cuda"), out, H, Hkv)
     torch.cuda.synchronize()
@@ -133,6 +141,8 @@ def test_attention_ranges_merged_in_kernel_over_many_calls(H, Hkv, hd, S):
     positions = torch.randint(0, S, (400,), generator=g, device="cuda").tolist()
     try:
         for i, pos in enumerate(positions):
+            if i == 100:
+                _lib.set_option("attention_single_below", 0)      # from here on every length is shared
             if i == 300:
                 _lib.set_option("attention_two_step", 1)
             q = (torch.randn(H * hd, generator=g, device="cuda") * 1.5).half()
@@ -142,6 +152,7 @@ def test_attention_ranges_merged_in_kernel_over_many_calls(H, Hkv, hd, S):
             assert _close(many, one, 3e-3), (i, pos)
     finally:
         _lib.set_option("attention_two_step", 0)
+        _lib.set_option("attention_single_below", 512)
     assert int(ws.view(torch.int32)[:H].abs().sum()) == 0
 
 
