@@ -262,6 +262,75 @@ def kernels_leg(torch, ext, F):
     return rows_out
 
 
+def helpers_leg(torch):
+    """Decode-step helper kernels, us per launch (graphs of back-to-back launches between HIP events): the dense output
+    head against torch's nn.Linear, and one-token attention at a range of positions in its two forms (a head's
+    positions shared by up to 8 workgroups / scanned by one workgroup)."""
+    from decdec_amd import _lib, decode_ops as D
+    from decdec_amd.model import rope_tables
+
+    def graph_time(fn, reps, iters):
+        st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            fn()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=st):
+            for _ in range(reps):
+                fn()
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (reps * iters)
+
+    out = {"dense_gemv": [], "rope_attention": [], "small": []}
+    for N, K in ((128256, 4096), (32064, 5120)):
+        w = (torch.randn(N, K, device="cuda") * 0.02).half()
+        x = torch.randn(K, device="cuda").half()
+        y = torch.empty(N, device="cuda", dtype=torch.float16)
+        lin = torch.nn.Linear(K, N, bias=False, device="cuda", dtype=torch.float16)
+        lin.weight.data = w
+        with torch.no_grad():
+            a = graph_time(lambda: D.dense_gemv(w, x, y), 20, 5)
+            b = graph_time(lambda: lin(x.view(1, 1, K)), 20, 5)
+        out["dense_gemv"].append({"N": N, "K": K, "us": round(a, 1), "gbs": round(N * K * 2 / a / 1e3, 1),
+                                  "frac_of_hbm_peak": round(N * K * 2 / a / 1e3 / 8000.0, 3), "torch_linear_us": round(b, 1)})
+        del w, lin
+    H, Hkv, hd, S = 32, 8, 128, 2048
+    cos, sin = rope_tables(hd, S, 10000.0, "cuda")
+    cos, sin = cos.half(), sin.half()
+    qkv = torch.randn((H + 2 * Hkv) * hd, device="cuda").half()
+    kc, vc = (torch.randn(1, Hkv, S, hd, device="cuda").half() for _ in range(2))
+    o = torch.empty(H * hd, device="cuda", dtype=torch.float16)
+    ws = D.attention_workspace(H, hd)
+    default = _lib.get_option("attention_single_below")
+    try:
+        for posv in (63, 255, 511, 640, 1023, 2047):
+            pos = torch.tensor([posv], device="cuda")
+            row = {"pos": posv}
+            for name, below in (("shared_us", 0), ("alone_us", S)):
+                _lib.set_option("attention_single_below", below)
+                row[name] = round(graph_time(lambda: D.rope_attention(qkv, cos, sin, pos, o, kc, vc, H, Hkv, ws), 100, 10), 2)
+            out["rope_attention"].append(row)
+    finally:
+        _lib.set_option("attention_single_below", default)
+    dim, inter = 4096, 14336
+    h, yv = (torch.randn(1, dim, device="cuda").half() for _ in range(2))
+    wn = torch.ones(dim, device="cuda", dtype=torch.float16)
+    ho, hn = torch.empty_like(h), torch.empty_like(h)
+    gu = torch.randn(2 * inter, device="cuda").half()
+    act = torch.empty(inter, device="cuda", dtype=torch.float16)
+    out["small"].append({"kernel": "add_rmsnorm 4096", "us": round(graph_time(lambda: D.add_rmsnorm(h, yv, wn, ho, hn, 1e-5), 200, 10), 2)})
+    out["small"].append({"kernel": "silu_mul 14336", "us": round(graph_time(lambda: D.silu_mul(gu, act), 200, 10), 2)})
+    return out
+
+
 def cpu_baseline_leg(protos, budget_s=15.0):
     """The same per-layer path (select + residual rows + any-precision GEMV) in the C oracle on the host
     cores, one layer of each shape, scaled to a token (32 layers)."""
@@ -301,9 +370,10 @@ def main():
     ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--leg", choices=["all", "roofline", "kernels"], default="all",
+    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers"], default="all",
                     help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
-                         "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 8)")
+                         "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 8); "
+                         "helpers: the decode harness's helper kernels (output head, attention, norm, activation)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
@@ -315,6 +385,9 @@ def main():
     _lib.load()
     torch.cuda.set_device(0)
 
+    if args.leg == "helpers":
+        print(json.dumps({"helpers": helpers_leg(torch)}))
+        return
     if args.leg == "kernels":
         print(json.dumps({"kernels": kernels_leg(torch, ext, F)}))
         return
