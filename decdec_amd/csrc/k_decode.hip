@@ -132,17 +132,11 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
     const uint32_t chunk = ((len + nsplit - 1u) / nsplit + 16u * PPW - 1u) / (16u * PPW) * (16u * PPW);
     const uint32_t lo = split * chunk < len ? split * chunk : len;
     const uint32_t hi = (lo + chunk) < len ? (lo + chunk) : len;
-    float q[8];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        q[2 * e] = E::from_raw(qr[e] & 0xFFFFu) * p.scale;
-        q[2 * e + 1] = E::from_raw(qr[e] >> 16) * p.scale;
-    }
     float m = -__builtin_inff(), l = 0.f, o[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = 0.f;
     // The scan is bound by the instruction issue of the workgroup's compute unit, so it is written to need few
-    // instructions: fp16 scores come from packed dot products of the raw registers (fp32 accumulation, scaled
+    // instructions: the scores come from packed dot products of the raw registers (fp32 accumulation, scaled
     // afterwards), and the UN rows of a trip share one update of the running maximum (one rescaling of the output
     // instead of UN).
     for (uint32_t p0 = lo + wave * PPW; p0 < hi; p0 += UN * 16 * PPW) {
@@ -160,23 +154,20 @@ __global__ __launch_bounds__(1024) void decode_attention_kernel(const AttentionP
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             float t = 0.f;
-            if constexpr (DT == kFP16) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t ka = kr[u][e], qb = qr[e];
+                if constexpr (DT == kFP16) {
                     half2_t a, b;
-                    const uint32_t ka = kr[u][e], qb = qr[e];
                     __builtin_memcpy(&a, &ka, 4); __builtin_memcpy(&b, &qb, 4);
                     t = __builtin_amdgcn_fdot2(a, b, t, false);
+                } else {
+                    bf16x2_t a, b;
+                    __builtin_memcpy(&a, &ka, 4); __builtin_memcpy(&b, &qb, 4);
+                    t = __builtin_amdgcn_fdot2_f32_bf16(a, b, t, false);
                 }
-                t = group_sum<LPP>(t) * p.scale;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    t += q[2 * e] * E::from_raw(kr[u][e] & 0xFFFFu);
-                    t += q[2 * e + 1] * E::from_raw(kr[u][e] >> 16);
-                }
-                t = group_sum<LPP>(t);
             }
+            t = group_sum<LPP>(t) * p.scale;
             const bool valid = p0 + (uint32_t)u * 16 * PPW + sub < hi;
             sc[u] = valid ? t : -__builtin_inff();
             mn = sc[u] > mn ? sc[u] : mn;
