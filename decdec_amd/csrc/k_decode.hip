@@ -315,27 +315,13 @@ __global__ __launch_bounds__(D) void decode_attention_merge_kernel(const Attenti
     E::store(p.out, (size_t)h * D + tid, Og / Lg);
 }
 
-// VEC = 4: n is a multiple of 4 and the tensors are 8-byte aligned (one 8-byte load of each half per thread)
-template <int DT, int VEC>
+template <int DT>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ gate_up, void* __restrict__ out, uint32_t n) {
     using E = Elem<DT>;
-    const uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * (uint32_t)VEC;
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    if constexpr (VEC == 4) {
-        const u32x2 ga = *(const u32x2*)((const uint16_t*)gate_up + i);
-        const u32x2 gb = *(const u32x2*)((const uint16_t*)gate_up + (size_t)n + i);
-        uint32_t r[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t sh = (e & 1) ? 16u : 0u;
-            const float a = E::from_raw((ga[e >> 1] >> sh) & 0xFFFFu), b = E::from_raw((gb[e >> 1] >> sh) & 0xFFFFu);
-            r[e] = E::to_raw(a / (1.f + __expf(-a)) * b) & 0xFFFFu;
-        }
-        *(u32x2*)((uint16_t*)out + i) = u32x2{r[0] | (r[1] << 16), r[2] | (r[3] << 16)};
-    } else {
-        const float a = E::load(gate_up, i), b = E::load(gate_up, (size_t)n + i);
-        E::store(out, i, a / (1.f + __expf(-a)) * b);
-    }
+    const float a = E::load(gate_up, i), b = E::load(gate_up, (size_t)n + i);
+    E::store(out, i, a / (1.f + __expf(-a)) * b);
 }
 
 // ---- dense 16-bit GEMV: the unquantised output head of a decoder ------------------------------------------
@@ -606,18 +592,10 @@ hipError_t launch_decode_attention(int dt, const AttentionParams& p, hipStream_t
 }
 
 hipError_t launch_silu_mul(int dt, const void* gate_up, void* out, uint32_t n, hipStream_t s) {
-    const bool vec = n % 4u == 0 && ((uintptr_t)gate_up % 8) == 0 && ((uintptr_t)out % 8) == 0;
-    const uint32_t threads = vec ? n / 4u : n;
-    const dim3 grid((threads + 255) / 256), block(256);
-    if (dt == kFP16) {
-        if (vec) hipLaunchKernelGGL((silu_mul_kernel<kFP16, 4>), grid, block, 0, s, gate_up, out, n);
-        else hipLaunchKernelGGL((silu_mul_kernel<kFP16, 1>), grid, block, 0, s, gate_up, out, n);
-    } else if (dt == kBF16) {
-        if (vec) hipLaunchKernelGGL((silu_mul_kernel<kBF16, 4>), grid, block, 0, s, gate_up, out, n);
-        else hipLaunchKernelGGL((silu_mul_kernel<kBF16, 1>), grid, block, 0, s, gate_up, out, n);
-    } else {
-        return hipErrorInvalidValue;
-    }
+    const dim3 grid((n + 255) / 256), block(256);
+    if (dt == kFP16) hipLaunchKernelGGL((silu_mul_kernel<kFP16>), grid, block, 0, s, gate_up, out, n);
+    else if (dt == kBF16) hipLaunchKernelGGL((silu_mul_kernel<kBF16>), grid, block, 0, s, gate_up, out, n);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 

@@ -174,7 +174,6 @@ def test_dense_gemv(N, K, dt):
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("n", [1, 12, 255, 1028, 14336, 17920])
 def test_silu_mul(n, dt):
-    """Multiples of 4 take the form with four outputs per thread, the others one output per thread."""
     gu = (torch.randn(2 * n, device="cuda") * 3).to(dt)
     out = torch.full((n,), 9.0, dtype=dt, device="cuda")
     D.silu_mul(gu, out)
