@@ -80,6 +80,45 @@ __device__ __forceinline__ float lutgemm_tiles(const LutgemmParams& p, uint32_t 
     return acc;
 }
 
+// The same walk with the requests of the next tile issued before the lookups of the current one, and the requests
+// of the first tile issued by the caller before the tables are built (they do not depend on the tables), so that
+// the first memory round trip of a wave runs behind the table build instead of after it.
+template <int DT, int BITS>
+struct LutgemmTile {
+    uint32_t w[BITS], araw[BITS], braw;
+};
+template <int DT, int BITS>
+__device__ __forceinline__ void lutgemm_issue(const LutgemmParams& p, uint32_t gt, uint32_t nc, LutgemmTile<DT, BITS>& r) {
+    using E = Elem<DT>;
+    const uint32_t g = (32u * gt) / p.group_size;
+#pragma unroll
+    for (int b = 0; b < BITS; ++b) {
+        r.w[b] = __builtin_nontemporal_load(p.qw + ((size_t)gt * BITS + b) * p.N + nc);
+        r.araw[b] = E::load_raw(p.alpha, ((size_t)g * BITS + b) * p.N + nc);
+    }
+    r.braw = E::load_raw(p.q_bias, (size_t)g * p.N + nc);
+}
+template <int DT, int BITS>
+__device__ __forceinline__ float lutgemm_tiles_ahead(const LutgemmParams& p, uint32_t t0, uint32_t lt0, uint32_t lt1,
+                                                     uint32_t nc, uint32_t tab_lds, const float* xsum,
+                                                     LutgemmTile<DT, BITS> cur) {
+    using E = Elem<DT>;
+    uint32_t m = 0x3Cu;
+    asm volatile("" : "+v"(m));                      // mask in a VGPR
+    float acc = 0.f;
+#pragma unroll 1
+    for (uint32_t lt = lt0; lt < lt1; ++lt) {
+        LutgemmTile<DT, BITS> nxt = cur;
+        if (lt + 1u < lt1) lutgemm_issue<DT, BITS>(p, t0 + lt + 1u, nc, nxt);     // uniform in the wave
+        const uint32_t tb = tab_lds + lt * 512u;
+        acc += E::from_raw(cur.braw) * xsum[lt];
+#pragma unroll
+        for (int b = 0; b < BITS; ++b) acc += E::from_raw(cur.araw[b]) * lutgemm_word(tb, cur.w[b], m);
+        cur = nxt;
+    }
+    return acc;
+}
+
 template <int DT>
 __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bid, unsigned char* smem) {
     using E = Elem<DT>;
@@ -95,6 +134,17 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
     float* tab = (float*)(smem + ((512u - (smem_lds & 511u)) & 511u));   // [wg_tiles][8][16]
     float* xsum = tab + (size_t)wg_tiles * 128;      // [wg_tiles]
     float* part = xsum + wg_tiles;                   // [nwaves][64]
+
+    const uint32_t n0 = nt * 64u, n = n0 + lane;
+    const bool col_ok = n < p.N;
+    const uint32_t nc = col_ok ? n : p.N - 1u;       // columns past the end re-read the last one
+    const uint32_t lt0 = wave * p.slice_tiles;       // local tiles of this wave: [lt0, lt1)
+    const uint32_t lt1 = (lt0 + p.slice_tiles) < nt_wg ? (lt0 + p.slice_tiles) : nt_wg;
+    // three planes (the usual format): the wave's first tile is requested before the tables exist
+    constexpr int kAhead = 3;
+    LutgemmTile<DT, kAhead> first = {};
+    const bool ahead = p.bits == (uint32_t)kAhead;
+    if (ahead && lt0 < lt1) lutgemm_issue<DT, kAhead>(p, t0 + lt0, nc, first);
 
     // tables: tab[(tile * 8 + j) * 16 + pat] = sum_i (bit i of pat ? +1 : -1) * x[32 tile + 4 j + i]
     for (uint32_t T = tid; T < nt_wg * 8u; T += nthreads) {
@@ -115,14 +165,10 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
     }
     __syncthreads();
 
-    const uint32_t n0 = nt * 64u, n = n0 + lane;
-    const bool col_ok = n < p.N;
-    const uint32_t nc = col_ok ? n : p.N - 1u;       // columns past the end re-read the last one
-    const uint32_t lt0 = wave * p.slice_tiles;       // local tiles of this wave: [lt0, lt1)
-    const uint32_t lt1 = (lt0 + p.slice_tiles) < nt_wg ? (lt0 + p.slice_tiles) : nt_wg;
     const uint32_t tab_lds = (uint32_t)(uintptr_t)(DD_LDS_AS float*)tab;    // LDS byte address of the tables
     float acc;
-    switch (p.bits) {
+    if (ahead) acc = lutgemm_tiles_ahead<DT, kAhead>(p, t0, lt0, lt1, nc, tab_lds, xsum, first);
+    else switch (p.bits) {
         case 1: acc = lutgemm_tiles<DT, 1>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
         case 2: acc = lutgemm_tiles<DT, 2>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
         case 3: acc = lutgemm_tiles<DT, 3>(p, t0, lt0, lt1, nc, tab_lds, xsum); break;
