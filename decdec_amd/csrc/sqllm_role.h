@@ -68,6 +68,13 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
     uint32_t lane4 = lane * 4u;
 
     if (p.bits == 4) {
+        // the first words of the wave's K range are requested before the table is built (they do not depend on it),
+        // and inside the loop the next words before the lookups of the current ones
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+        if (k0 < k1) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(k0 / 8u + u) * p.N);
+        }
         // build: this thread's column, high field = wave, low field 0..15
         {
             const u32x4 a = *(const u32x4*)lrow, b = *(const u32x4*)(lrow + 8);
@@ -84,9 +91,11 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
         asm volatile("" : "+v"(m), "+v"(lane4));
 #pragma unroll 1
         for (uint32_t c = k0; c < k1; c += 32u) {
-            uint32_t w[4];
+            uint32_t wn[4] = {w[0], w[1], w[2], w[3]};
+            if (c + 32u < k1) {                                  // uniform in the wave
 #pragma unroll
-            for (int u = 0; u < 4; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(c / 8u + u) * p.N);
+                for (int u = 0; u < 4; ++u) wn[u] = __builtin_nontemporal_load(col + (size_t)((c + 32u) / 8u + u) * p.N);
+            }
             uint32_t xd[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) xd[i] = xs[(c >> 1) + i];
@@ -99,8 +108,15 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
                     acc = sqllm_dot2<DT>(pr, xd[4 * u + k], acc);
                 }
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) w[u] = wn[u];
         }
     } else {
+        uint32_t w[3] = {0u, 0u, 0u};                            // requested ahead, as in the 4-bit path
+        if (k0 < k1) {
+#pragma unroll
+            for (int u = 0; u < 3; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(3u * (k0 / 32u) + u) * p.N);
+        }
         // 3-bit: 64 entries; high field = wave / 2, low fields 4 (wave & 1) .. + 3
         {
             const u32x4 a = *(const u32x4*)lrow;
@@ -118,9 +134,11 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
         asm volatile("" : "+v"(m), "+v"(lane4));
 #pragma unroll 1
         for (uint32_t c = k0; c < k1; c += 32u) {
-            uint32_t w[3];
+            uint32_t wn[3] = {w[0], w[1], w[2]};
+            if (c + 32u < k1) {                                  // uniform in the wave
 #pragma unroll
-            for (int u = 0; u < 3; ++u) w[u] = __builtin_nontemporal_load(col + (size_t)(3u * (c / 32u) + u) * p.N);
+                for (int u = 0; u < 3; ++u) wn[u] = __builtin_nontemporal_load(col + (size_t)(3u * ((c + 32u) / 32u) + u) * p.N);
+            }
             uint32_t xd[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) xd[i] = xs[(c >> 1) + i];
@@ -134,6 +152,8 @@ __device__ __forceinline__ void sqllm_role_pairs(const SqllmParams& p, uint32_t 
                 const uint32_t pr = *(const uint32_t*)(lt + ((v & m) | lane4));
                 acc = sqllm_dot2<DT>(pr, xd[k], acc);
             }
+#pragma unroll
+            for (int u = 0; u < 3; ++u) w[u] = wn[u];
         }
     }
     part[wave * 64u + lane] = acc;
