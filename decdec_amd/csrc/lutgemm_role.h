@@ -146,7 +146,8 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
     const bool ahead = p.bits == (uint32_t)kAhead;
     if (ahead && lt0 < lt1) lutgemm_issue<DT, kAhead>(p, t0 + lt0, nc, first);
 
-    // tables: tab[(tile * 8 + j) * 16 + pat] = sum_i (bit i of pat ? +1 : -1) * x[32 tile + 4 j + i]
+    // tables: tab[(tile * 8 + j) * 16 + pat] = sum_i (bit i of pat ? +1 : -1) * x[32 tile + 4 j + i]; the eight tables
+    // of a tile are built by eight neighbouring lanes, which also add up the tile's plain sum (the factor of q_bias)
     for (uint32_t T = tid; T < nt_wg * 8u; T += nthreads) {
         const size_t c0 = (size_t)32 * t0 + (size_t)4 * T;
         const float x0 = E::load(p.x, c0), x1 = E::load(p.x, c0 + 1), x2 = E::load(p.x, c0 + 2), x3 = E::load(p.x, c0 + 3);
@@ -155,13 +156,11 @@ __device__ __forceinline__ void lutgemm_role(const LutgemmParams& p, uint32_t bi
         float* dst = tab + (size_t)T * 16;
 #pragma unroll
         for (int q = 0; q < 16; ++q) dst[q] = lo[q & 3] + hi[q >> 2];
-    }
-    __syncthreads();
-    for (uint32_t t = tid; t < nt_wg; t += nthreads) {
-        float s = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s += tab[(size_t)(t * 8 + j) * 16 + 15];
-        xsum[t] = s;
+        float sx = lo[3] + hi[3];
+        sx += __shfl_xor(sx, 1, 64);
+        sx += __shfl_xor(sx, 2, 64);
+        sx += __shfl_xor(sx, 4, 64);
+        if ((T & 7u) == 0u) xsum[T >> 3] = sx;
     }
     __syncthreads();
 
