@@ -60,6 +60,7 @@ struct Options {
     int attention_single_below = 512;  // ... and merging in the kernel: sequences up to this length are not shared at all
     int fused_small = -1;       // fused 3-bit any-precision launches with both roles in the GEMV's own smaller workgroups:
                                 // -1 = when those have 5..8 waves (measured faster there), 1 = whenever they have <= 8, 0 = never
+    int dec_max_chunk_groups = 0;  // DEC launch plans: at most this many chunk groups (atomic adds per output); 0 = the built-in bound
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
@@ -87,6 +88,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "attention_two_step")) return &g_opt.attention_two_step;
     if (!strcmp(name, "attention_single_below")) return &g_opt.attention_single_below;
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
+    if (!strcmp(name, "dec_max_chunk_groups")) return &g_opt.dec_max_chunk_groups;
     return nullptr;
 }
 
@@ -242,30 +244,44 @@ Config* get_config(uint64_t h) {
 
 constexpr size_t kLdsBudget = 60 * 1024;
 
+// Upper bound on the chunk groups of a DEC launch.  Every chunk group adds its partial sum to an output with an
+// atomic add of its own, i.e. one more rounding of a 16-bit output in an order that varies from run to run; the
+// reference adds once per output (dec.cu:263-276).  With 14 of them (K = 14336) an output now and then missed the
+// 1e-2 bound.  A workgroup selects up to (waves / 4) chunks at a time, so few chunk groups cost little.
+constexpr uint32_t kMaxChunkGroups = 4;
+
 // Split the DEC work of one layer over at most `budget` workgroups of `nw` waves: cg chunk groups x sg
-// segment groups, minimising the longest per-workgroup path; ties prefer fewer chunk groups (= fewer atomic
-// adds per output).  The row list of a workgroup must fit in LDS.
+// segment groups, cg <= kMaxChunkGroups (option dec_max_chunk_groups can lower it), minimising the longest
+// per-workgroup path; ties prefer fewer chunk groups.  The row list of a workgroup must fit in LDS: only a
+// row list that fits with no allowed cg (k_chunk in the hundreds at K > 16384) lifts the bound.
 int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t nw, DecPlan* pl) {
     const uint32_t num_chunks = cdiv(K, 1024);
     const uint32_t nseg = cdiv(M, 64);
+    const uint32_t teams = std::max(1u, nw / 4u);
     budget = std::max(1u, budget);
+    uint32_t cap = kMaxChunkGroups;
+    if (g_opt.dec_max_chunk_groups >= 1) cap = std::min(cap, (uint32_t)g_opt.dec_max_chunk_groups);
     uint64_t best_cost = ~0ull;
     uint32_t best_cg = 0, best_sg = 0;
     size_t best_lds = 0;
-    for (uint32_t cg = 1; cg <= num_chunks; ++cg) {
-        const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
-        for (uint32_t sg = 1; sg <= sg_max; ++sg) {
-            const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
-            const uint32_t slots = (cpb * std::max(k_chunk, 1u) + 1u) & ~1u;   // even: keeps the LDS arrays behind the row list 16-byte aligned
-            const size_t lds = dec_lds_bytes(slots, nw);
-            if (lds > kLdsBudget) continue;
-            // per-workgroup critical path: sequential chunk selections, then batches of eight rows per
-            // wave for each group of up to nw segments; going over the workgroup budget is a last resort
-            const uint32_t sb = std::min(spb, nw), rl = nw / sb;
-            const uint64_t batches = (uint64_t)cdiv(spb, nw) * cdiv(slots, rl * 8);
-            const uint64_t cost = batches * 1000 + (uint64_t)cpb * 600 + (uint64_t)cg * 10 +
-                                  (cg * sg > budget ? 500000ull : 0);
-            if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
+    for (int pass = 0; pass < 2 && best_cg == 0; ++pass) {
+        const uint32_t cg_max = pass == 0 ? std::min(num_chunks, cap) : num_chunks;
+        for (uint32_t cg = 1; cg <= cg_max; ++cg) {
+            const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
+            for (uint32_t sg = 1; sg <= sg_max; ++sg) {
+                const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
+                const uint32_t slots = (cpb * std::max(k_chunk, 1u) + 1u) & ~1u;   // even: keeps the LDS arrays behind the row list 16-byte aligned
+                const size_t lds = dec_lds_bytes(slots, nw);
+                if (lds > kLdsBudget) continue;
+                // per-workgroup critical path: rounds of selection (one chunk per team of four waves), then
+                // batches of eight rows per wave for each group of up to nw segments; going over the
+                // workgroup budget is a last resort
+                const uint32_t sb = std::min(spb, nw), rl = nw / sb;
+                const uint64_t batches = (uint64_t)cdiv(spb, nw) * cdiv(slots, rl * 8);
+                const uint64_t cost = batches * 1000 + (uint64_t)cdiv(cpb, teams) * 600 + (uint64_t)cg * 10 +
+                                      (cg * sg > budget ? 500000ull : 0);
+                if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
+            }
         }
     }
     if (best_cg == 0) return 1;
@@ -347,6 +363,8 @@ int check_dec_call(const Config* c, int dtype, uint32_t in_features, uint32_t ou
     DD_CHECK(out_features == c->N, "output tensor size does not match with DECConfig: output size: %u, DECConfig size: %u",
              out_features, c->N);
     DD_CHECK(c->ctx != nullptr && c->ctx->dt == c->dt, "Data type mismatch between DECConfig and DECContext.");
+    // 16-bit outputs are merged with packed two-element atomic adds on even element pairs
+    DD_CHECK(dtype == DECDEC_FP32 || ((uintptr_t)output % 4) == 0, "output must be 4-byte aligned");
     return kOk;
 }
 
@@ -418,6 +436,7 @@ int plan_lutgemm(const void* input, void* output, const void* qw, const void* al
     DD_CHECK(group_size >= 32 && group_size % 32 == 0 && K % (uint32_t)group_size == 0,
              "group_size must be a multiple of 32 that divides input_feat, got %d", group_size);
     DD_CHECK(N >= 1, "output_feat must be positive");
+    DD_CHECK(((uintptr_t)output % 4) == 0, "output must be 4-byte aligned");
     LutgemmParams& p = pl->p;
     memset(&p, 0, sizeof(p));
     p.x = input; p.qw = (const uint32_t*)qw; p.alpha = alpha; p.q_bias = q_bias; p.out = output;
@@ -466,6 +485,7 @@ int plan_sqllm(const void* input, void* output, const void* mat, const void* lut
     DD_CHECK(input && output && mat && lut, "null pointer argument");
     DD_CHECK(K >= 32 && K % 32 == 0, "input_feat must be a positive multiple of 32, got %u", K);
     DD_CHECK(N >= 1, "output_feat must be positive");
+    DD_CHECK(((uintptr_t)output % 4) == 0, "output must be 4-byte aligned");
     SqllmParams& p = pl->p;
     memset(&p, 0, sizeof(p));
     p.x = input; p.mat = (const uint32_t*)mat; p.lut = lut; p.out = output;
@@ -630,6 +650,10 @@ int decdec_destroy_dec_context(uint64_t h) {
     DD_CHECK(c != nullptr, "invalid DECContext handle");
     {
         std::lock_guard<std::mutex> l(g_mu);
+        // a config keeps a pointer to its context: destroying a context that live configs use would leave it dangling
+        for (uint64_t ch : g_configs)
+            if (reinterpret_cast<Config*>(ch)->ctx == c)
+                return fail(kInvalid, "DECContext is still used by a DECConfig; destroy or update the config first");
         g_contexts.erase(h);
     }
     (void)hipStreamDestroy(c->sub_stream);

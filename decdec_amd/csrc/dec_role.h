@@ -53,10 +53,18 @@ constexpr int kMaxCand = 256;                                // fast-path candid
 constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per thread and segment batch
 
 __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves = kDecWaves) {
-    // row list (index + activation) + selection counters/prefix + the buffer shared by the cross-wave
-    // reduction ([nwaves][8][64] floats) and the partial ranks of the selection ([16][kMaxCand] bytes)
-    const size_t red = (size_t)nwaves * 8 * kWave * 4, ranks = (size_t)16 * kMaxCand;
-    return (size_t)slots * 8 + 2 * 512 * 4 + (red > ranks ? red : ranks);
+    // row list (index + activation) + counters/prefix of the general selection + the buffer shared by the
+    // cross-wave reduction ([nwaves][8][64] floats) and the selection teams (one area per four waves)
+    const size_t red = (size_t)nwaves * 8 * kWave * 4;
+    const size_t teams = (size_t)(nwaves / 4) * ((size_t)(32 + 2 * kMaxCand + 8) * 4 + (size_t)16 * kMaxCand);
+    return (size_t)slots * 8 + 2 * 512 * 4 + (red > teams ? red : teams);
+}
+
+// The 32 bucket floors live in one vector register (lane i and lane i + 32 hold floor[i], read from the kernel
+// argument segment once per workgroup) and are broadcast with v_readlane where they are used: as 32 scalar kernel
+// arguments they would be held in scalar registers for the whole kernel.
+__device__ __forceinline__ float dec_floor(float myfloor, int i) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
 }
 
 // ---- selection of one chunk ------------------------------------------------------------------
@@ -66,7 +74,7 @@ __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves 
 template <int DT, int NW>
 __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t c, uint32_t t_local, uint32_t kc,
                                                 int32_t* lrows, float* lacts, uint32_t* cnt, uint32_t* pre,
-                                                bool write_global) {
+                                                bool write_global, const float myfloor) {
     using E = Elem<DT>;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     constexpr uint32_t nw = NW;
@@ -78,7 +86,6 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
     // read again and its memberships recomputed (this path is rare; registers held here would be charged to
     // every launch of the kernels that contain it).
     const uint32_t ngroups = (uint32_t)(kChunk / kWave);
-    const float myfloor = p.floors[lane & 31u];                      // lane i holds floor[i]
 #pragma unroll 1
     for (uint32_t vw = wave; vw < ngroups; vw += nw) {
         const uint32_t ch = vw * kWave + lane;
@@ -88,7 +95,7 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
         float ce = __builtin_inff();
 #pragma unroll 1
         for (int i = 0; i < kBuckets; ++i) {
-            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+            const float fl = dec_floor(myfloor, i);
             const bool bit = (a >= fl) && (a < ce);
             ce = fl;
             const unsigned long long m = __ballot(bit);
@@ -121,7 +128,7 @@ __device__ __forceinline__ void dec_select_general(const DecParams& p, uint32_t 
 #pragma unroll 1
         for (int i = 0; i < kBuckets; ++i) {
             if (pre[i * 16] >= kc) break;                            // uniform: later buckets start even later
-            const float fl = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
+            const float fl = dec_floor(myfloor, i);
             const bool bit = (a >= fl) && (a < ce);
             ce = fl;
             const unsigned long long m = __ballot(bit);
@@ -157,17 +164,33 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // range they are the only possible picks.  Eight cut-offs T are tried at once (a compare and a ballot
 // each); the first whose range holds at least kc and at most kMaxCand channels wins.  Those candidates
 // (usually a few dozen of 1024) are compacted in channel order, get the key (bucket << 10 | channel),
-// and the canonical position of a candidate is the number of smaller keys, counted all-pairs in tiles of
-// 64 candidates x 16 keys spread over the waves.  No sequential walk over buckets.
+// and the canonical position of a candidate is the number of smaller keys, counted all-pairs.  No
+// sequential walk over buckets.
 //
-// A wave issues one instruction every four cycles whatever its kind, and an instruction issued by all
-// 16 waves of the workgroup occupies each SIMD four times as long; so the scan of the 1024 channels is
-// done by four waves (one per SIMD, four channels per lane) while the others wait at the barrier, and
-// the candidate phases only involve the waves that hold candidates or tiles.
+// A wave issues one instruction every four cycles whatever its kind, so a chunk is scanned by a TEAM of
+// four waves (one per SIMD, four channels per lane).  The teams of a workgroup (four in a 1024-thread
+// workgroup) take different chunks of the workgroup's chunk list at the same time: a workgroup that owns
+// up to four chunks selects them in the time of one, which is what lets the launch plan give a workgroup
+// several chunks (few chunk groups = few atomic adds, i.e. roundings, per output) at no cost in latency.
+// All teams run through the same workgroup barriers; what a team does between them depends on its own
+// chunk only.  A chunk the fast path cannot take (non-monotone floors, more than kMaxCand candidates,
+// k_chunk > kMaxCand) is afterwards selected by the whole workgroup on the general path.
 constexpr int kAttempts = 8;
-constexpr int kSelWaves = 4;
+constexpr int kSelWaves = 4;                                 // waves of a team
+constexpr int kTeamThreads = kSelWaves * kWave;
+// per-team LDS: candidate counts [kAttempts][kSelWaves], keys [kMaxCand], activations [kMaxCand], header
+// (state, candidate count; padded), partial ranks [16][kMaxCand] bytes
+constexpr int kTeamWords = 32 + 2 * kMaxCand + 8;
+constexpr size_t kTeamBytes = (size_t)kTeamWords * 4 + (size_t)16 * kMaxCand;
+enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u };
+
 __device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) {
     return u == 0 ? 15u : u == 1 ? 18u : u == 2 ? 21u : u == 3 ? 23u : u == 4 ? 25u : u == 5 ? 27u : u == 6 ? 29u : 31u;
+}
+// the same for a wave-uniform run-time attempt number: one byte per attempt
+__device__ __forceinline__ uint32_t dec_attempt_bucket_rt(uint32_t u) {
+    const unsigned long long tab = 0x1F1D1B191715120Full;   // bytes 15, 18, 21, 23, 25, 27, 29, 31
+    return (uint32_t)(tab >> (8u * u)) & 0xFFu;
 }
 
 // The four activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
@@ -179,29 +202,51 @@ __device__ __forceinline__ void dec_load_x4(const DecParams& p, uint32_t lo, uin
     for (int s = 0; s < 4; ++s) xr[s] = Elem<DT>::load_raw(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
 }
 
+__device__ __forceinline__ uint32_t dec_chunk_len(const DecParams& p, uint32_t c) {
+    const uint32_t lo = c * kChunk;
+    return (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
+}
+
+// One round of selection: team j of the workgroup takes the workgroup's local chunk t0 + j (global chunk
+// cgid + (t0 + j) * cg) if there is one.  `xpre` holds the raw activations of the team's chunk when
+// have_xpre (requested when the workgroup started).  Called by all threads of the workgroup.
 template <int DT, int NW>
-__device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c, uint32_t t_local,
+__device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cgid, uint32_t t0, uint32_t nlocal,
                                                  int32_t* lrows, float* lacts, uint32_t* cnt,
                                                  uint32_t* pre, float* red, bool write_global,
-                                                 bool have_xpre, const uint32_t (&xpre)[4]) {
+                                                 bool have_xpre, const uint32_t (&xpre)[4], const float myfloor) {
     using E = Elem<DT>;
+    constexpr uint32_t kTeams = NW / kSelWaves;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t lo = c * kChunk;
-    const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
+    const uint32_t team = wave / (uint32_t)kSelWaves, tw = wave % (uint32_t)kSelWaves;
+    const uint32_t ttid = tid & (uint32_t)(kTeamThreads - 1);
+    const uint32_t t_local = t0 + team;
+    const uint32_t c = cgid + t_local * p.cg;
+    const bool has_chunk = t_local < nlocal;                // uniform per wave
+    const uint32_t lo = has_chunk ? c * kChunk : 0u;
+    const uint32_t len = has_chunk ? dec_chunk_len(p, c) : 0u;
     const uint32_t kc = p.k_chunk * len / kChunk;
-    if (kc == 0) return;                                   // uniform for the workgroup
+    const bool active = has_chunk && kc > 0u;
 
-    uint32_t* wc = cnt;                                    // [kAttempts][kSelWaves] candidate counts
-    uint32_t* key = cnt + 32;                              // [kMaxCand]
-    float* cx = (float*)(cnt + 32 + kMaxCand);             // [kMaxCand] (runs into `pre`, unused here)
-    uint32_t* hdr = cnt + 32 + 2 * kMaxCand;               // fast flag, candidate count
-    uint8_t* pc = (uint8_t*)red;                           // [16][kMaxCand] partial ranks (each at most 16)
-    const bool scanner = p.monotone && wave < (uint32_t)kSelWaves;   // uniform per wave
+    unsigned char* tbase = (unsigned char*)red + (size_t)team * kTeamBytes;
+    uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][kSelWaves] candidate counts
+    uint32_t* key = wc + 32;                               // [kMaxCand]
+    float* cx = (float*)(key + kMaxCand);                  // [kMaxCand]
+    uint32_t* hdr = key + 2 * kMaxCand;                    // state, candidate count
+    uint8_t* pc = tbase + (size_t)kTeamWords * 4;          // [16][kMaxCand] partial ranks (each at most 16)
+    const bool scanner = active && p.monotone;             // uniform per wave
 
-    // ---- four waves scan the chunk: lane l of wave w owns channels 4 (64 w + l) .. + 3
-    float xv[4], a[4];
-    const uint32_t ch0 = 4u * tid;
+    // ---- the team scans its chunk: lane l of team wave w owns channels 4 (64 w + l) .. + 3
+    // |x| of the lane's channel s as the selection sees it: NaN, inf and channels past the end are members of no
+    // bucket.  Recomputed after the barrier instead of kept: registers held across it are charged to every kernel
+    // that contains this role.
+    float xv[4];
+    const uint32_t ch0 = 4u * ttid;
+    auto mag = [&](int s) {
+        const float v = __builtin_fabsf(xv[s]);
+        return (ch0 + (uint32_t)s < len && v < __builtin_inff()) ? v : -__builtin_inff();
+    };
     if (scanner) {
         uint32_t xr[4];
         if (have_xpre) {                                   // uniform: requested when the workgroup started
@@ -213,67 +258,70 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
         asm volatile("" : "+v"(xr[0]), "+v"(xr[1]), "+v"(xr[2]), "+v"(xr[3]));   // first use: here
 #pragma unroll
         for (int s = 0; s < 4; ++s) xv[s] = E::from_raw(xr[s]);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const bool in = ch0 + s < len;
-            const float v = __builtin_fabsf(xv[s]);
-            a[s] = (in && v < __builtin_inff()) ? v : -__builtin_inff();   // NaN, inf: members of no bucket
-        }
         dec_stamp(p, blockIdx.x, 5);
         uint32_t n[kAttempts];
+        {
+            float a[4];
 #pragma unroll
-        for (int u = 0; u < kAttempts; ++u) {
-            const float f = p.floors[dec_attempt_bucket(u)];
-            n[u] = 0;
+            for (int s = 0; s < 4; ++s) a[s] = mag(s);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) n[u] += (uint32_t)__popcll(__ballot(a[s] >= f));
+            for (int u = 0; u < kAttempts; ++u) {
+                const float f = dec_floor(myfloor, (int)dec_attempt_bucket(u));
+                n[u] = 0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) n[u] += (uint32_t)__popcll(__ballot(a[s] >= f));
+            }
         }
         if (lane == 0) {
 #pragma unroll
-            for (int u = 0; u < kAttempts; ++u) wc[u * kSelWaves + wave] = n[u];
+            for (int u = 0; u < kAttempts; ++u) wc[u * kSelWaves + tw] = n[u];
         }
     }
     __syncthreads();
     if (scanner) {
-        // lane u < 8 looks at attempt u: total and the count of the waves before this one
+        // lane u < 8 looks at attempt u: total and the count of the team's waves before this one
         const u32x4 w4 = *(const u32x4*)(wc + kSelWaves * (lane & 7u));
         const uint32_t tot = w4[0] + w4[1] + w4[2] + w4[3];
-        const uint32_t before = (wave > 0 ? w4[0] : 0u) + (wave > 1 ? w4[1] : 0u) + (wave > 2 ? w4[2] : 0u);
+        const uint32_t before = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
         const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= (uint32_t)kMaxCand);
         const bool fast = okm != 0ull;
         if (fast) {
             const uint32_t us = (uint32_t)__builtin_ctzll(okm);                     // first qualifying attempt
             const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)us);
             const uint32_t base = (uint32_t)__builtin_amdgcn_readlane((int)before, (int)us);
-            const float f = p.floors[dec_attempt_bucket(us)];
+            const float f = dec_floor(myfloor, (int)dec_attempt_bucket_rt(us));
             uint32_t cs[4], mine = 0;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) { cs[s] = (a[s] >= f) ? 1u : 0u; mine += cs[s]; }
+            for (int s = 0; s < 4; ++s) { cs[s] = (mag(s) >= f) ? 1u : 0u; mine += cs[s]; }
             uint32_t idx = base + wave_scan(mine) - mine;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
             }
-            if (tid == 0) hdr[1] = total;
+            if (ttid == 0) hdr[1] = total;
         }
-        if (tid == 0) hdr[0] = fast ? 1u : 0u;
-    } else if (!p.monotone && tid == 0) {
-        hdr[0] = 0u;
+        if (ttid == 0) hdr[0] = fast ? kTeamFast : kTeamGeneral;
+    } else if (ttid == 0) {
+        hdr[0] = active ? kTeamGeneral : kTeamIdle;
+        hdr[1] = 0u;
     }
     __syncthreads();
-    const u32x2 hd = *(const u32x2*)hdr;
-    if (hd[0] == 0u) {                                     // uniform
-        __syncthreads();                                   // hdr is read before cnt is reused
-        dec_select_general<DT, NW>(p, c, t_local, kc, lrows, lacts, cnt, pre, write_global);
-        return;
+    // what the teams found (the same view in every thread: the branches below that hold barriers are uniform)
+    bool any_big = false, any_general = false;
+#pragma unroll
+    for (uint32_t j = 0; j < kTeams; ++j) {
+        const u32x2 h = *(const u32x2*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)(32 + 2 * kMaxCand) * 4);
+        any_general = any_general || h[0] == kTeamGeneral;
+        any_big = any_big || (h[0] == kTeamFast && h[1] > (uint32_t)kWave);
     }
+    const u32x2 hd = *(const u32x2*)hdr;
+    const bool fast = hd[0] == kTeamFast;
     const uint32_t total = hd[1];
     dec_stamp(p, blockIdx.x, 6);
-    if (total <= (uint32_t)kWave) {
+    if (fast && total <= (uint32_t)kWave) {
         // The usual case: at most 64 candidates.  One wave holds a candidate per lane and ranks them all-pairs
-        // against the key list read back as broadcasts; nothing here needs a workgroup barrier (the other
-        // waves go straight to the barrier that precedes the fetch).
-        if (wave == 0) {
+        // against the key list read back as broadcasts; nothing here needs a workgroup barrier.
+        if (tw == 0) {
             uint32_t mykey = 0xFFFFFFFFu;                  // padding: never smaller than a real key
             float xs = 0.f;
             if (lane < total) {
@@ -281,7 +329,7 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
                 const float ca = __builtin_fabsf(xs);
                 uint32_t bkt = 0;
 #pragma unroll
-                for (int i = 0; i < kBuckets; ++i) bkt += (ca < p.floors[i]) ? 1u : 0u;
+                for (int i = 0; i < kBuckets; ++i) bkt += (ca < dec_floor(myfloor, i)) ? 1u : 0u;
                 mykey = (bkt << 10) | key[lane];
             }
             key[lane] = mykey;
@@ -308,58 +356,70 @@ __device__ __forceinline__ void dec_select_chunk(const DecParams& p, uint32_t c,
                 }
             }
         }
-        dec_stamp(p, blockIdx.x, 7);
-        return;
     }
-    // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
-    if (__builtin_amdgcn_readfirstlane(tid & ~63u) < total) {
-        if (tid < total) {
-            const float ca = __builtin_fabsf(cx[tid]);
-            uint32_t bkt = 0;
+    if (any_big) {                                         // uniform for the workgroup
+        const bool big = fast && total > (uint32_t)kWave;  // uniform per team
+        // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
+        if (big && __builtin_amdgcn_readfirstlane(ttid & ~63u) < total) {
+            if (ttid < total) {
+                const float ca = __builtin_fabsf(cx[ttid]);
+                uint32_t bkt = 0;
 #pragma unroll
-            for (int i = 0; i < kBuckets; ++i) bkt += (ca < p.floors[i]) ? 1u : 0u;
-            key[tid] |= bkt << 10;
-        } else if (tid < ((total + 15u) & ~15u)) {
-            key[tid] = 0xFFFFFFFFu;                        // padding of the last 16-key tile: never smaller
-        }
-    }
-    __syncthreads();
-    {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per wave and round
-        const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
-#pragma unroll 1
-        for (uint32_t tile = wave; tile < ntiles; tile += (uint32_t)NW) {
-            const uint32_t jg = tile % njg, iq = tile / njg;
-            const uint32_t j = jg * 64u + lane;
-            const uint32_t mykey = j < total ? key[j] : 0u;
-            const u32x4* kp = (const u32x4*)(key + iq * 16u);
-            uint32_t r = 0;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const u32x4 k4 = kp[v];
-                r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
+                for (int i = 0; i < kBuckets; ++i) bkt += (ca < dec_floor(myfloor, i)) ? 1u : 0u;
+                key[ttid] |= bkt << 10;
+            } else if (ttid < ((total + 15u) & ~15u)) {
+                key[ttid] = 0xFFFFFFFFu;                   // padding of the last 16-key tile: never smaller
             }
-            pc[iq * kMaxCand + j] = (uint8_t)r;
         }
-    }
-    __syncthreads();
-    if (__builtin_amdgcn_readfirstlane(tid & ~63u) < total && tid < total) {
-        const uint32_t niq = (total + 15u) >> 4;
-        uint32_t pos = 0;
+        __syncthreads();
+        if (big) {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per team wave and step
+            const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
+#pragma unroll 1
+            for (uint32_t tile = tw; tile < ntiles; tile += (uint32_t)kSelWaves) {
+                const uint32_t jg = tile % njg, iq = tile / njg;
+                const uint32_t j = jg * 64u + lane;
+                const uint32_t mykey = j < total ? key[j] : 0u;
+                const u32x4* kp = (const u32x4*)(key + iq * 16u);
+                uint32_t r = 0;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const u32x4 k4 = kp[v];
+                    r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
+                }
+                pc[iq * kMaxCand + j] = (uint8_t)r;
+            }
+        }
+        __syncthreads();
+        if (big && __builtin_amdgcn_readfirstlane(ttid & ~63u) < total && ttid < total) {
+            const uint32_t niq = (total + 15u) >> 4;
+            uint32_t pos = 0;
 #pragma unroll 4
-        for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kMaxCand + tid];
-        if (pos < kc) {
-            const uint32_t ch = lo + (key[tid] & 1023u);
-            const float xs = cx[tid];
-            const uint32_t slot = t_local * p.k_chunk + pos;
-            lrows[slot] = (int32_t)ch;
-            lacts[slot] = xs;
-            if (write_global) {
-                p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
-                E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
+            for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kMaxCand + ttid];
+            if (pos < kc) {
+                const uint32_t ch = lo + (key[ttid] & 1023u);
+                const float xs = cx[ttid];
+                const uint32_t slot = t_local * p.k_chunk + pos;
+                lrows[slot] = (int32_t)ch;
+                lacts[slot] = xs;
+                if (write_global) {
+                    p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
+                    E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
+                }
             }
         }
     }
     dec_stamp(p, blockIdx.x, 7);
+    if (any_general) {                                     // uniform for the workgroup; rare
+#pragma unroll 1
+        for (uint32_t j = 0; j < kTeams; ++j) {
+            const uint32_t st = *(const uint32_t*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)(32 + 2 * kMaxCand) * 4);
+            if (st != kTeamGeneral) continue;              // uniform
+            const uint32_t tj = t0 + j, cj = cgid + tj * p.cg;
+            const uint32_t kcj = p.k_chunk * dec_chunk_len(p, cj) / kChunk;
+            __syncthreads();                               // cnt / pre of the previous general selection no longer read
+            dec_select_general<DT, NW>(p, cj, tj, kcj, lrows, lacts, cnt, pre, write_global, myfloor);
+        }
+    }
 }
 
 // ---- fetch + dequantise + accumulate ------------------------------------------------------------
@@ -482,24 +542,26 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
     float* red = (float*)(pre + 512);
 
     dec_stamp(p, bid, 0);
-    // the scanning waves ask for the activations of the workgroup's first chunk before anything else: their
-    // latency is the head of the critical path
+    // the teams ask for the activations of their first chunks before anything else: their latency is the
+    // head of the critical path
+    constexpr uint32_t kTeams = (uint32_t)NW / kSelWaves;
+    const uint32_t nlocal = cgid < p.num_chunks ? (p.num_chunks - cgid + p.cg - 1u) / p.cg : 0u;   // chunks cgid, cgid + cg, ...
+    const float myfloor = p.floors[tid & 31u];
     uint32_t xpre[4] = {0u, 0u, 0u, 0u};
-    const bool have_xpre = p.fused_select && p.monotone && cgid < p.num_chunks;      // uniform
-    if (have_xpre && tid < (uint32_t)kSelWaves * kWave) {
-        const uint32_t lo = cgid * kChunk;
-        const uint32_t len = (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
-        dec_load_x4<DT>(p, lo, len, 4u * tid, xpre);
+    const uint32_t team0 = tid / (uint32_t)kTeamThreads;
+    const bool have_xpre = p.fused_select && p.monotone;                              // uniform
+    if (have_xpre && team0 < nlocal) {
+        const uint32_t c = cgid + team0 * p.cg;
+        dec_load_x4<DT>(p, c * kChunk, dec_chunk_len(p, c), 4u * (tid & (uint32_t)(kTeamThreads - 1)), xpre);
     }
     for (uint32_t i = tid; i < p.slots_per_block; i += (uint32_t)NW * kWave) lrows[i] = -1;
     uint32_t nslots = 0;
     if (p.fused_select) {
-        uint32_t t = 0;
-        for (uint32_t c = cgid; c < p.num_chunks; c += p.cg, ++t) {
-            __syncthreads();      // list initialised; cnt/pre of the previous chunk no longer read
-            dec_select_chunk<DT, NW>(p, c, t, lrows, lacts, cnt, pre, red, sgid == 0, have_xpre && t == 0, xpre);
+        for (uint32_t t0 = 0; t0 < nlocal; t0 += kTeams) {
+            __syncthreads();      // list initialised; the team areas of the previous round no longer read
+            dec_select_round<DT, NW>(p, cgid, t0, nlocal, lrows, lacts, cnt, pre, red, sgid == 0, have_xpre && t0 == 0, xpre, myfloor);
         }
-        nslots = t * p.k_chunk;
+        nslots = nlocal * p.k_chunk;
     } else {
         const uint32_t per = (p.k_total + p.cg - 1) / p.cg;
         const uint32_t lo = cgid * per;

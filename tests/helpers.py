@@ -47,3 +47,17 @@ def rel_err(got: np.ndarray, want: np.ndarray, floor: float = REL_FLOOR):
     got = got.astype(np.float64); want = want.astype(np.float64)
     denom = np.maximum(np.abs(want), floor * np.max(np.abs(want)) + 1e-30)
     return float(np.max(np.abs(got - want) / denom)), float(np.mean(np.abs(got - want)))
+
+
+TOL = {"fp16": 1e-2, "fp32": 1e-2, "bf16": 8e-2}     # bf16 has 8 significand bits against fp16's 11: the same bound in ulps
+
+
+def check_output(got: np.ndarray, want: np.ndarray, dt: str = "fp16", what=None) -> float:
+    """Asserts the output tolerance and reports, beside the judged ratio (10 % floor), the mean absolute error and
+    the same ratio with the denominator floored at 1 % of max|want|."""
+    mre, mae = rel_err(got, want)
+    strict, _ = rel_err(got, want, floor=0.01)
+    msg = f"{what}: max rel err {mre:.3e} (bound {TOL[dt]:.0e}), mean abs err {mae:.3e}, with a 1 % floor {strict:.3e}"
+    print(msg)
+    assert mre <= TOL[dt], msg
+    return mre

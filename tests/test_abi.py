@@ -89,12 +89,45 @@ def test_dec_launch_plan_covers_the_layer(waves):
                     assert 1 <= cg <= chunks and 1 <= sg <= nseg and info.hip_dec_blocks == cg * sg
                     cpb, spb = -(-chunks // cg), -(-nseg // sg)
                     assert info.hip_slots_per_block >= cpb * k_chunk and info.hip_slots_per_block % 2 == 0
-                    red = max(waves * 2048, 16 * 256)
+                    red = max(waves * 2048, (waves // 4) * ((32 + 512 + 8) * 4 + 16 * 256))
                     assert info.hip_lds_bytes == info.hip_slots_per_block * 8 + 4096 + red <= 60 * 1024
                     budget = n_tb * (16 // waves)
                     assert cg * sg <= budget or cg == 1 or chunks > budget, (K, N, n_tb, k_chunk, cg, sg)
                     if k_chunk <= 32 and budget >= chunks * -(-nseg // waves):
                         assert spb <= waves, (K, N, n_tb, k_chunk, cg, sg)
+
+
+MAX_CHUNK_GROUPS = 4
+
+CONFIG_SHAPES = [(4096, 4096), (4096, 1024), (4096, 14336), (14336, 4096), (4096, 6144), (4096, 28672),      # Llama-3-8B
+                 (5120, 7680), (5120, 5120), (5120, 35840), (17920, 5120),                                   # Phi-3-medium
+                 (8192, 8192), (8192, 1024), (8192, 28672), (28672, 8192)]                                   # Llama-3-70B
+
+
+@pytest.mark.parametrize("waves", [4, 8, 16])
+def test_dec_launch_plan_bounds_the_atomic_adds_per_output(waves):
+    """Every chunk group of a DEC launch adds its partial sum to an output with one atomic add (one more rounding of a
+    16-bit output, in run-to-run varying order); the reference adds once (dec.cu:263-276).  The plan keeps the chunk
+    groups within a small bound at every configuration shape, workgroup size and workgroup budget."""
+    lib = _lib.load()
+    info = _lib.ConfigInfo()
+    for K, N in CONFIG_SHAPES:
+        for n_tb in (8, 16, 32, 64):
+            for k_chunk in (1, 8, 16, 32, 64):
+                _lib.check(lib.decdec_dec_launch_plan(K, N, n_tb, k_chunk, waves, ctypes.byref(info)))
+                assert 1 <= info.hip_chunk_groups <= MAX_CHUNK_GROUPS, (K, N, n_tb, k_chunk, info.hip_chunk_groups)
+                assert info.hip_dec_blocks <= max(n_tb * (16 // waves), info.hip_chunk_groups)
+    # the option lowers the bound (1 = the reference's single add per output)
+    _lib.set_option("dec_max_chunk_groups", 1)
+    try:
+        for K, N in CONFIG_SHAPES:
+            _lib.check(lib.decdec_dec_launch_plan(K, N, 32, 32, waves, ctypes.byref(info)))
+            assert info.hip_chunk_groups == 1
+    finally:
+        _lib.set_option("dec_max_chunk_groups", 0)
+    # only a row list that cannot fit in LDS otherwise lifts the bound (select-all at a 70B input width)
+    _lib.check(lib.decdec_dec_launch_plan(28672, 8192, 32, 1024, waves, ctypes.byref(info)))
+    assert info.hip_chunk_groups > MAX_CHUNK_GROUPS and info.hip_lds_bytes <= 60 * 1024
 
 
 def test_invalid_handles_and_arguments_fail_cleanly():
