@@ -52,6 +52,7 @@ SIGNATURES = {
     "decdec_dummy_sqllm": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
     "decdec_rope_cache_update": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp],
     "decdec_decode_attention": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp, _u64, _vp],
+    "decdec_decode_attention_static": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp],
     "decdec_rope_attention": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _vp, _u64, _vp],
     "decdec_dense_gemv": [_vp, _vp, _vp, _i32, _u32, _u32, _vp],
     "decdec_silu_mul": [_vp, _vp, _i32, _u32, _vp],

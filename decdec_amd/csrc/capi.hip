@@ -18,6 +18,12 @@
 
 using namespace decdec;
 
+// Device memory that is part of the library image (see decdec_decode_attention_static): [heads] arrival counters,
+// then [heads][8][head_dim + 2] floats, at the largest supported size.
+constexpr uint32_t kStaticHeads = 128, kStaticHeadDim = 128, kStaticSplits = 8;
+constexpr size_t kStaticScratchBytes = (size_t)kStaticHeads * 4u + (size_t)kStaticHeads * kStaticSplits * (kStaticHeadDim + 2) * 4u;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 enum { kOk = 0, kInvalid = 1, kHipError = 2, kUnsupported = 3 };
@@ -556,6 +562,32 @@ static int dummy_common(int dummy_cu, int64_t iters, hipStream_t main_stream, Ge
     return kOk;
 }
 
+// ---- the static workspace of decdec_decode_attention_static ------------------------------------------------
+// Every GPU the library runs on holds its own copy of `scratch` at its own address; host code never uses the
+// array's name as a pointer, only the address hipGetSymbolAddress returns with that device current.
+
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void** out) {
+    int dev = -1;
+    DD_HIP(hipGetDevice(&dev));
+    DD_CHECK(dev >= 0 && dev < kMaxDevices, "device index %d is outside the supported range", dev);
+    std::lock_guard<std::mutex> l(g_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        DD_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+        DD_CHECK(ptr != nullptr, "hipGetSymbolAddress returned a null address for the static workspace");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return kOk;
+}
+
+__global__ __launch_bounds__(128) void fill_u32_kernel(uint32_t* dst, uint32_t n, uint32_t value) {
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = value;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1038,9 +1070,9 @@ int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void*
     return kOk;
 }
 
-int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
-                            void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
-                            uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
+static int decode_attention_common(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                                   void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                                   uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
     DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
     DD_CHECK(q && k_cache && v_cache && pos_device && out, "null pointer argument");
     DD_CHECK(n_head >= 1 && n_kv_head >= 1 && n_head % n_kv_head == 0, "n_head must be a multiple of n_kv_head");
@@ -1061,6 +1093,33 @@ int decdec_decode_attention(const void* q, const void* k_cache, const void* v_ca
                       (uint32_t)std::max(0, g_opt.attention_single_below)};
     DD_HIP(launch_decode_attention(dtype, p, (hipStream_t)stream));
     return kOk;
+}
+
+int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                            void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                            uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
+    return decode_attention_common(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
+                                   workspace, workspace_bytes, stream);
+}
+
+int decdec_decode_attention_static(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                                   void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                                   uint32_t max_seq, void* stream) {
+    DD_CHECK(n_head <= kStaticHeads, "decdec_decode_attention_static: n_head %u exceeds the limit of %u heads", n_head,
+             kStaticHeads);
+    DD_CHECK(head_dim <= kStaticHeadDim, "decdec_decode_attention_static: head_dim %u exceeds the limit of %u", head_dim,
+             kStaticHeadDim);
+    void* ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc != kOk) return rc;
+    // The array keeps what the last call left.  Every call leaves the counters at zero; clearing the ones this call
+    // uses makes that independent of what ran before (a fill kernel, not a memset node: safe under capture).
+    if (n_head >= 1) {
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(128), 0, (hipStream_t)stream, (uint32_t*)ws, n_head, 0u);
+        DD_HIP(hipGetLastError());
+    }
+    return decode_attention_common(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
+                                   ws, kStaticScratchBytes, stream);
 }
 
 int decdec_rope_attention(const void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos_device,

@@ -51,6 +51,19 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                                                    workspace.numel() * 4 if workspace is not None else 0, _stream()))
 
 
+def decode_attention_static(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pos: torch.Tensor,
+                            out: torch.Tensor, n_head: int, n_kv_head: int) -> None:
+    """`decode_attention` with the library's own static workspace: nothing is allocated and no workspace is passed
+    (at most 128 heads; calls on one GPU must not overlap in time)."""
+    _half_cuda(q, k_cache, v_cache, out)
+    _check(pos.is_cuda and pos.dtype == torch.int64 and pos.numel() == 1, "pos must be one int64 on the device")
+    D, max_seq = k_cache.shape[-1], k_cache.shape[-2]
+    _check(q.numel() == n_head * D and out.numel() == n_head * D, "q / out size mismatch")
+    _check(k_cache.numel() == n_kv_head * max_seq * D and v_cache.shape == k_cache.shape, "cache shape mismatch")
+    _lib.check(_lib.load().decdec_decode_attention_static(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(pos), _ptr(out),
+                                                          _dt(q), n_head, n_kv_head, D, max_seq, _stream()))
+
+
 def rope_attention(qkv: torch.Tensor, cos_table: torch.Tensor, sin_table: torch.Tensor, pos: torch.Tensor,
                    out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, n_head: int, n_kv_head: int,
                    workspace: torch.Tensor | None = None) -> None:

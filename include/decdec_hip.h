@@ -63,7 +63,9 @@ int decdec_version(void);
  * "attention_two_step" (decode attention with a workspace: 1 = merge in a second kernel, 0 = in the kernel [default]),
  * "attention_single_below" (... merging in the kernel: sequences of at most this many positions are scanned by one
  * workgroup per head, which is faster there; default 512, 0 = always share),
- * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows), "dec_trace" (see
+ * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows),
+ * "dec_max_chunk_groups" (DEC launch plans made from now on use at most this many chunk groups, i.e. atomic adds per
+ * output: 1 to 4; 0 = the built-in bound of 4 [default]), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
 int decdec_get_option(const char* name, int* value);
@@ -197,6 +199,17 @@ int decdec_rope_attention(const void* qkv, const void* cos_table, const void* si
                           const int64_t* pos_device, void* out, void* k_cache, void* v_cache, int dtype,
                           uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq,
                           void* workspace, uint64_t workspace_bytes, void* stream);
+/* decdec_decode_attention for callers that cannot allocate or own a workspace (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same kernels and the same result, with the workspace (arrival
+ * counters and partial results of the shared heads) held in a device array that is part of the library image --
+ * 532,992 bytes on every GPU the library runs on, until the process ends.  Limits: n_head <= 128, head_dim 64 or 128;
+ * anything larger is refused with an error.  The call allocates nothing; it clears the counters it uses with a small
+ * fill kernel and then launches the attention kernel on `stream`.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on one GPU (two streams, two threads) race.  The first call on a device looks the
+ * array's address up and must not run under stream capture.  No counterpart in the reference. */
+int decdec_decode_attention_static(const void* q, const void* k_cache, const void* v_cache,
+                                   const int64_t* pos_device, void* out, int dtype, uint32_t n_head,
+                                   uint32_t n_kv_head, uint32_t head_dim, uint32_t max_seq, void* stream);
 int decdec_dense_gemv(const void* weight, const void* x, void* out, int dtype, uint32_t N, uint32_t K,
                       void* stream);
 int decdec_silu_mul(const void* gate_up, void* out, int dtype, uint32_t n, void* stream);
