@@ -11,10 +11,18 @@ back to back through the C ABI.  The step is captured once in a HIP graph (the r
 loop runs under CUDA graphs as well, end-to-end/generate.py:115-121) and replayed; every replayed
 kernel is the library's own.  The activations, weights and residuals are synthetic (seeded).
 
-Prints ONE JSON line.  `value` = us/token with DEC (k_chunk 32, n_tb 8); `base_us_per_token` and
+Inside a decoder layer q, k and v read the same activation vector, and so do gate and up: the step runs each of
+these groups as ONE launch (decdec_dec_anyprec_batch; every layer of a group with a DEC context of its own), o and
+down as launches of their own -- 4 launches per decoder layer, the dependencies a decoder has.
+`serial_us_per_token` is the same work as 224 single-layer launches back to back, `graph_branches_us_per_token`
+the single-layer launches with q | k | v and gate | up as parallel branches of the captured graph.
+
+Prints ONE JSON line.  `value` = us/token with DEC (k_chunk 32, n_tb 32 by default); `base_us_per_token` and
 `dec_slowdown_pct` sit beside it; `roofline` is the any-precision GEMV of the largest layer shape
-(4096 -> 14336) measured with HIP events on its own stream; `cpu_baseline` is the C restatement of
-the same layer path (oracle/decdec_oracle.c, OpenMP over the host cores) on a bounded sample.
+(4096 -> 14336) measured with HIP events on its own stream, next to a plain read of the same bytes;
+`roofline_link` is the fused DEC + GEMV launch of that shape against the host link, next to a plain zero-copy
+read of pinned memory (the measured ceiling of the link); `cpu_baseline` is the C restatement of the same
+layer path (oracle/decdec_oracle.c, OpenMP over the host cores) on a bounded sample, all cores and one thread.
 """
 from __future__ import annotations
 
@@ -100,10 +108,76 @@ def time_graph(torch, graph, steps, warmup):
     return (time.perf_counter() - t0) / steps * 1e6
 
 
-# HBM traffic of one launch of the roofline kernel, bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --leg roofline`, each scaled by what the same counter reads for the 256 MiB device copy that the
-# leg also runs (profiles/anyprec_gemv_4096x14336_pmc.md holds the runs); None = not measured for this build
-MEASURED_TRAFFIC = {"anyprec_kernel<fp16,3> 4096->14336": 23122000}
+def measured_traffic():
+    """HBM traffic of one launch of the roofline kernel, bytes, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+    `bench.py --leg roofline`, each scaled by what the same counter reads for the 256 MiB device copy that the leg
+    also runs.  Read from the line `traffic_bytes_per_launch: N` of the profile summary that holds those runs;
+    None when the file or the line is missing."""
+    path = os.path.join(ROOT, "profiles", "anyprec_gemv_4096x14336_pmc.md")
+    try:
+        for line in open(path):
+            if line.strip().startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1].split()[0])
+    except (OSError, ValueError):
+        pass
+    return None
+
+
+def event_time_us(torch, stream, graph, reps):
+    """Average microseconds per replay of `graph`, HIP events on the stream the graph is launched on."""
+    with torch.cuda.stream(stream):
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        for _ in range(reps):
+            graph.replay()
+        b.record(stream)
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / reps
+
+
+def read_probe(torch, srcs, row_bytes, rows, vec_words, blocks, scramble, iters=5):
+    """Microseconds per launch of the library's plain read kernel over `rows` rows of `row_bytes` bytes; one launch
+    per tensor of `srcs` in a captured graph (distinct memory per launch, so that no launch is served from a cache
+    the previous one warmed)."""
+    from decdec_amd import _lib
+    lib = _lib.load()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+
+    def launches():
+        for t in srcs:
+            _lib.check(lib.decdec_debug_read_probe(t.data_ptr(), row_bytes, rows, vec_words, blocks, int(scramble),
+                                                   sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    with torch.cuda.stream(stream):
+        launches()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        launches()
+    g.replay()
+    torch.cuda.synchronize()
+    return event_time_us(torch, stream, g, iters) / len(srcs)
+
+
+def link_leg(torch, full=False):
+    """Ceiling of zero-copy reads of pinned host memory: the library's plain read kernel over a pinned buffer, rows
+    of the residual's row size visited in scattered order, for a range of workgroup counts and request widths."""
+    nbuf = 4
+    per = (16 << 20) if full else (8 << 20)               # per launch: long enough to be bandwidth-bound
+    bufs = [torch.empty(per // 4, dtype=torch.int32, pin_memory=True) for _ in range(nbuf)]
+    for b in bufs:
+        b.random_(0, 1 << 20)
+    out = []
+    cases = [(rb, vec, blocks) for rb in ((2048, 7168) if full else (7168,)) for vec in ((1, 2, 4) if full else (1, 4))
+             for blocks in ((8, 16, 32, 64, 128) if full else (32, 64))]
+    for rb, vec, blocks in cases:
+        rows = per // rb
+        us = read_probe(torch, bufs, rb, rows, vec, blocks, True, iters=3)
+        out.append({"row_bytes": rb, "vec_words": vec, "blocks": blocks, "bytes": rows * rb, "us": round(us, 1),
+                    "GBs": round(rows * rb / us / 1e3, 2)})
+    return out
 
 
 def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
@@ -131,15 +205,13 @@ def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
     g.replay()
     torch.cuda.synchronize()
     reps = max(1, iters // ncopy)
-    with torch.cuda.stream(stream):
-        a = torch.cuda.Event(enable_timing=True)
-        b = torch.cuda.Event(enable_timing=True)
-        a.record(stream)
-        for _ in range(reps):
-            g.replay()
-        b.record(stream)
-    torch.cuda.synchronize()
-    us = a.elapsed_time(b) * 1e3 / (reps * ncopy)
+    us = event_time_us(torch, stream, g, reps) / ncopy
+    # a plain read of the same number of bytes with as many waves as the GEMV launches (nothing but loads): what
+    # a launch of this size can reach at all on this memory system
+    by_w = BITS * N * K // 8
+    srcs = [c.view(-1) for c in copies]
+    stream_us = min(read_probe(torch, srcs, 4096, by_w // 4096, vec, blocks, False, iters=3)
+                    for vec, blocks in ((1, 680), (2, 340), (4, 170), (4, 340), (4, 512)))
     if calibrate_copy:      # known-size device copy for scaling the FETCH_SIZE / WRITE_SIZE counters
         src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device="cuda")
         dst = torch.empty_like(src)
@@ -151,7 +223,49 @@ def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
     name = "anyprec_kernel<fp16,3> 4096->14336"
     return {"bound": "hbm", "kernel": name, "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": MEASURED_TRAFFIC.get(name)}
+            "us_per_launch": round(us, 3), "bytes_per_launch": by, "traffic": measured_traffic(),
+            "plain_read_us": round(stream_us, 3), "plain_read_frac": round(by_w / stream_us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def roofline_link_leg(torch, ext, protos, k_chunk, n_tb, link_table):
+    """The dominant kernel of the timed step: the fused DEC + GEMV launch on 4096 -> 14336, whose duration is set by
+    the residual rows it reads over the host link (k_chunk * K / 1024 rows of N / 2 bytes).  HIP events on the launch
+    stream over private weight and residual copies; beside it the best rate of the plain zero-copy read kernel."""
+    K, N = 4096, 14336
+    p = protos[(K, N)]
+    ncopy = 12
+    copies = [p["qweight"].clone() for _ in range(ncopy)]
+    x = torch.randn(1, 1, K, dtype=torch.float16, device="cuda")
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    rows = torch.zeros(K, dtype=torch.int32, device="cuda")
+    acts = torch.zeros(K, dtype=torch.float16, device="cuda")
+    ctx = ext.create_dec_context(n_tb, rows, acts)
+    cfgs = [ext.create_dec_config(ctx, k_chunk, p["cheat"], p["scales"], p["th"]) for _ in range(ncopy)]
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+
+    def launches():
+        for i in range(ncopy):
+            ext.dec_anyprec(cfgs[i], x, out, copies[i], p["lut"], BITS)
+    with torch.cuda.stream(stream):
+        launches()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=stream):
+        launches()
+    g.replay()
+    torch.cuda.synchronize()
+    us = event_time_us(torch, stream, g, 10) / ncopy
+    for c in cfgs:
+        ext.destroy_dec_config(c)
+    ext.destroy_dec_context(ctx)
+    by = (k_chunk * K // 1024) * (N // 2)
+    achieved = by / us / 1e3
+    ceiling = max(r["GBs"] for r in link_table)
+    return {"bound": "host link (PCIe Gen5 x16)", "kernel": f"dec_anyprec_kernel<fp16,3> {K}->{N}, k_chunk {k_chunk}, n_tb {n_tb}",
+            "bytes_per_launch": by, "us_per_launch": round(us, 3), "achieved": round(achieved, 2), "peak": 64.0,
+            "unit": "GB/s", "frac": round(achieved / 64.0, 4), "measured_ceiling": ceiling,
+            "frac_of_measured_ceiling": round(achieved / ceiling, 4), "plain_read": link_table}
 
 
 def kernels_leg(torch, ext, F):
@@ -331,33 +445,53 @@ def helpers_leg(torch):
     return out
 
 
-def cpu_baseline_leg(protos, budget_s=15.0):
-    """The same per-layer path (select + residual rows + any-precision GEMV) in the C oracle on the host
-    cores, one layer of each shape, scaled to a token (32 layers)."""
+def cpu_baseline_leg(protos, iters=20, budget_s=25.0):
+    """The same per-layer path (select + residual rows + any-precision GEMV) in the C oracle on the host cores: one
+    layer of each shape, median of `iters` warmed calls, scaled to a token (32 layers); with all cores and with
+    one thread (fewer iterations if the time budget runs out)."""
     import numpy as np
     from oracle import c_oracle
     c_oracle.build()
+    c_oracle.lib()
     cores = os.cpu_count() or 1
-    os.environ.setdefault("OMP_NUM_THREADS", str(min(cores, 64)))
+    try:
+        omp = ctypes.CDLL("libgomp.so.1")
+    except OSError:
+        omp = None
     rng = np.random.default_rng(0)
-    per_shape = {}
-    t_start = time.perf_counter()
+    data = {}
     for (K, N), p in protos.items():
-        x = rng.standard_normal(K).astype(np.float16)
-        qw = p["qweight"].cpu().numpy(); lut = p["lut"].cpu().numpy()
-        cheat = p["cheat"].numpy(); sc = p["scales"].numpy(); th = p["th"].numpy().astype(np.float32)
-        k = 32 * K // 1024
-        t0 = time.perf_counter()
-        c_oracle.layer_anyprec_dec(x, qw, lut, BITS, cheat, sc, float(th[0]), float(th[k - 1]), 32)
-        per_shape[(K, N)] = (time.perf_counter() - t0) * 1e6
-        if time.perf_counter() - t_start > budget_s:
-            break
-    if len(per_shape) < len(protos):
-        return None
-    token_us = 32 * sum(per_shape[(K, N)] for _, K, N in LLAMA3_8B)
-    return {"value": round(token_us, 1), "unit": "us/token", "cores": int(os.environ["OMP_NUM_THREADS"]),
-            "kind": "port", "sample": "one DEC-compensated layer of each of the 4 Llama-3-8B shapes (C oracle, "
-            "OpenMP, float64 accumulate), x32 layers with q/o, k/v and gate/up counted twice"}
+        th = p["th"].numpy().astype(np.float32)
+        data[(K, N)] = (rng.standard_normal(K).astype(np.float16), p["qweight"].cpu().numpy(), p["lut"].cpu().numpy(),
+                        p["cheat"].numpy(), p["scales"].numpy(), float(th[0]), float(th[32 * K // 1024 - 1]))
+
+    def token_us(threads, deadline):
+        if omp is not None:
+            omp.omp_set_num_threads(int(threads))
+        per_shape, n_done = {}, iters
+        for (K, N), (x, qw, lut, cheat, sc, ta, tb) in data.items():
+            for _ in range(2):                                    # warm-up
+                c_oracle.layer_anyprec_dec(x, qw, lut, BITS, cheat, sc, ta, tb, 32)
+            ts = []
+            for _ in range(iters):
+                t0 = time.perf_counter()
+                c_oracle.layer_anyprec_dec(x, qw, lut, BITS, cheat, sc, ta, tb, 32)
+                ts.append((time.perf_counter() - t0) * 1e6)
+                if time.perf_counter() > deadline and len(ts) >= 3:
+                    break
+            per_shape[(K, N)] = float(np.median(ts))
+            n_done = min(n_done, len(ts))
+        return 32 * sum(per_shape[(K, N)] for _, K, N in LLAMA3_8B), n_done
+
+    t0 = time.perf_counter()
+    all_us, n_all = token_us(cores, t0 + budget_s * 0.35)
+    one_us, n_one = (token_us(1, t0 + budget_s) if omp is not None else (None, 0))
+    if omp is not None:
+        omp.omp_set_num_threads(int(cores))
+    return {"value": round(all_us, 1), "unit": "us/token", "cores": int(cores if omp is not None else 1), "kind": "port",
+            "sample": f"one DEC-compensated layer of each of the 4 Llama-3-8B shapes (C oracle, OpenMP, float64 accumulate), "
+                      f"median of {n_all} warmed calls per shape, x32 layers with q/o, k/v and gate/up counted twice",
+            "one_thread_value": None if one_us is None else round(one_us, 1), "one_thread_iters": n_one}
 
 
 def main():
@@ -370,10 +504,11 @@ def main():
     ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers"], default="all",
+    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers", "link"], default="all",
                     help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
-                         "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 8); "
-                         "helpers: the decode harness's helper kernels (output head, attention, norm, activation)")
+                         "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 32); "
+                         "helpers: the decode harness's helper kernels (output head, attention, norm, activation); "
+                         "link: zero-copy reads of pinned host memory over workgroup counts and request widths")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
@@ -388,6 +523,9 @@ def main():
     if args.leg == "helpers":
         print(json.dumps({"helpers": helpers_leg(torch)}))
         return
+    if args.leg == "link":
+        print(json.dumps({"link": link_leg(torch, full=True)}))
+        return
     if args.leg == "kernels":
         print(json.dumps({"kernels": kernels_leg(torch, ext, F)}))
         return
@@ -397,29 +535,88 @@ def main():
         return
     layers, xs, protos, arena = build_layer_set(torch, F, args.layers, args.k_chunk, seed=0)
     maxK = max(l["K"] for l in layers)
-    rows = torch.zeros(maxK, dtype=torch.int32, device="cuda")
-    acts = torch.zeros(maxK, dtype=torch.float16, device="cuda")
+
+    NAMES = [n for n, _, _ in LLAMA3_8B]
+    # q, k, v share an input and are independent, and so are gate and up: branch 0 (the main one) runs q, o, gate,
+    # down; branch 1 runs k and up; branch 2 runs v.  Launches that overlap in time must not share a DEC context
+    # (its scratch buffers), so every branch has one.
+    BRANCH = {"q": 0, "k": 1, "v": 2, "o": 0, "gate": 0, "up": 1, "down": 0}
+    scratch = [(torch.zeros(maxK, dtype=torch.int32, device="cuda"), torch.zeros(maxK, dtype=torch.float16, device="cuda"))
+               for _ in range(3)]
+    side = [torch.cuda.Stream(), torch.cuda.Stream()]
 
     def make_configs(n_tb, k_chunk):
-        ctx = ext.create_dec_context(n_tb, rows, acts)
-        return ctx, [ext.create_dec_config(ctx, k_chunk, l["cheat"], l["scales"], l["th"]) for l in layers]
+        ctxs = [ext.create_dec_context(n_tb, r, a) for r, a in scratch]
+        return ctxs, [ext.create_dec_config(ctxs[BRANCH[l["name"]]], k_chunk, l["cheat"], l["scales"], l["th"]) for l in layers]
 
-    def base_step():
+    def drop_configs(ctxs, cfgs):
+        for c in cfgs:
+            ext.destroy_dec_config(c)
+        for c in ctxs:
+            ext.destroy_dec_context(c)
+
+    def run_step(launch, mode, batch=None):
+        """One token.  launch(i) enqueues linear i on the current stream; batch(ids) enqueues the linears `ids` (which
+        share an input) as one launch.  mode "batched": q | k | v and gate | up are one launch each (4 launches per
+        decoder layer); "branches": one launch per linear, q | k | v and gate | up as parallel branches of the captured
+        graph; "serial": one launch per linear, back to back."""
         arena.zero_()
-        for l in layers:
-            ext.anyprec_gemv(xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+        if mode == "serial":
+            for i in range(len(layers)):
+                launch(i)
+            return
+        main_s = torch.cuda.current_stream()
+        for base_i in range(0, len(layers), len(NAMES)):
+            idx = {n: base_i + j for j, n in enumerate(NAMES)}
+            if mode == "batched":
+                batch([idx["q"], idx["k"], idx["v"]])
+                launch(idx["o"])
+                batch([idx["gate"], idx["up"]])
+                launch(idx["down"])
+                continue
+            for st in side:
+                st.wait_stream(main_s)
+            launch(idx["q"])
+            with torch.cuda.stream(side[0]):
+                launch(idx["k"])
+            with torch.cuda.stream(side[1]):
+                launch(idx["v"])
+            for st in side:
+                main_s.wait_stream(st)
+            launch(idx["o"])
+            side[0].wait_stream(main_s)
+            launch(idx["gate"])
+            with torch.cuda.stream(side[0]):
+                launch(idx["up"])
+            main_s.wait_stream(side[0])
+            launch(idx["down"])
 
-    ctx, cfgs = make_configs(args.n_tb, args.k_chunk)
+    def base_launch(i):
+        l = layers[i]
+        ext.anyprec_gemv(xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
 
-    def dec_step():
-        arena.zero_()
-        for l, c in zip(layers, cfgs):
-            ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+    def base_batch(ids):
+        ls = [layers[i] for i in ids]
+        ext.dec_anyprec_batch(None, xs[ls[0]["K"]], [l["out"] for l in ls], [l["qweight"] for l in ls], [l["lut"] for l in ls], BITS)
 
-    g_base = capture(torch, base_step)
-    g_dec = capture(torch, dec_step)
-    base_us = time_graph(torch, g_base, args.steps, args.warmup)
-    dec_us = time_graph(torch, g_dec, args.steps, args.warmup)
+    ctxs, cfgs = make_configs(args.n_tb, args.k_chunk)
+
+    def dec_launch(i):
+        l = layers[i]
+        ext.dec_anyprec(cfgs[i], xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
+
+    def dec_batch(ids):
+        ls = [layers[i] for i in ids]
+        ext.dec_anyprec_batch([cfgs[i] for i in ids], xs[ls[0]["K"]], [l["out"] for l in ls], [l["qweight"] for l in ls],
+                              [l["lut"] for l in ls], BITS)
+
+    times = {}
+    for name, launch, batch in (("base", base_launch, base_batch), ("dec", dec_launch, dec_batch)):
+        for mode in ("batched", "serial", "branches"):
+            g = capture(torch, lambda: run_step(launch, mode, batch))
+            times[(name, mode)] = time_graph(torch, g, args.steps, args.warmup)
+            del g
+    base_us, dec_us = times[("base", "batched")], times[("dec", "batched")]
     scale = 32.0 / args.layers
 
     # clearing the outputs is part of the layer contract (the kernels accumulate), so the arena fill stays
@@ -436,32 +633,32 @@ def main():
         "config": {"workload": "configs[1]: Llama-3-8B decoder linear shapes, batch 1, any-precision 3-bit base "
                    "from HBM, 4-bit residuals in pinned host memory", "layers": args.layers,
                    "linears_per_layer": 7, "k_chunk": args.k_chunk, "n_tb": args.n_tb, "fusion": "single launch",
-                   "graph_replay": True},
+                   "graph_replay": True, "launches_per_decoder_layer": 4,
+                   "batched_launches": "q|k|v in one launch, o, gate|up in one launch, down"},
         "base_us_per_token": round(base_us * scale, 2),
         "dec_slowdown_pct": round((dec_us / base_us - 1) * 100, 2),
+        "serial_us_per_token": round(times[("dec", "serial")] * scale, 2),
+        "serial_base_us_per_token": round(times[("base", "serial")] * scale, 2),
+        "serial_dec_slowdown_pct": round((times[("dec", "serial")] / times[("base", "serial")] - 1) * 100, 2),
+        "graph_branches_us_per_token": round(times[("dec", "branches")] * scale, 2),
+        "graph_branches_base_us_per_token": round(times[("base", "branches")] * scale, 2),
         "zero_fill_us_per_token": round(zero_us * scale, 2),
         "base_hbm_gbs": round(weight_bytes / (base_us - zero_us) / 1e3, 1),
         "dec_host_link_bytes_per_token": int(host_bytes * scale),
+        "dec_host_link_gbs": round(host_bytes / dec_us / 1e3, 2),
     }
-    for c in cfgs:
-        ext.destroy_dec_config(c)
-    ext.destroy_dec_context(ctx)
+    result["roofline_link"] = roofline_link_leg(torch, ext, protos, args.k_chunk, args.n_tb, link_leg(torch))
+    drop_configs(ctxs, cfgs)
 
     if args.sweep:
         sweep = []
         for n_tb in (8, 16, 32, 64):
             for k_chunk in (8, 16, 32, 64):
-                ctx, cfgs = make_configs(n_tb, k_chunk)
-                def step():
-                    arena.zero_()
-                    for l, c in zip(layers, cfgs):
-                        ext.dec_anyprec(c, xs[l["K"]], l["out"], l["qweight"], l["lut"], BITS)
-                us = time_graph(torch, capture(torch, step), max(5, args.steps // 2), 2)
+                ctxs, cfgs = make_configs(n_tb, k_chunk)
+                us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2)
                 sweep.append({"n_tb": n_tb, "k_chunk": k_chunk, "us_per_token": round(us * scale, 1),
                               "slowdown_pct": round((us / base_us - 1) * 100, 1)})
-                for c in cfgs:
-                    ext.destroy_dec_config(c)
-                ext.destroy_dec_context(ctx)
+                drop_configs(ctxs, cfgs)
         result["sweep"] = sweep
 
     result["roofline"] = roofline_leg(torch, ext, protos)

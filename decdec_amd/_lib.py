@@ -45,6 +45,8 @@ SIGNATURES = {
     "decdec_lutgemm_gemv": [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _u32, _u32, _vp],
     "decdec_sqllm_gemv": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _vp],
     "decdec_dec_anyprec": [_u64, _vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _vp],
+    "decdec_dec_anyprec_batch": [_u32, ctypes.POINTER(_u64), _vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                                 ctypes.POINTER(_vp), _i32, _i32, _u32, ctypes.POINTER(_u32), _vp],
     "decdec_dec_lutgemm": [_u64, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _u32, _u32, _vp],
     "decdec_dec_sqllm": [_u64, _vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _vp],
     "decdec_dummy_anyprec": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
@@ -59,6 +61,7 @@ SIGNATURES = {
     "decdec_add_rmsnorm": [_vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp],
     "decdec_greedy_pick": [_vp, _u32, _i32, _vp, _vp, _vp, _vp, _u32, _vp, _vp, _vp],
     "decdec_debug_read_trace": [ctypes.POINTER(_u64), _i32],
+    "decdec_debug_read_probe": [_vp, _u64, _u64, _u32, _u32, _i32, _vp, _vp],
     "decdec_bucket_floors": [_f32, _f32, _i32, ctypes.POINTER(_f32)],
     "decdec_reference_geometry": [_u32, _u32, _u32, _u32, _i32, _u32, ctypes.POINTER(ConfigInfo)],
     "decdec_dec_launch_plan": [_u32, _u32, _u32, _u32, _u32, ctypes.POINTER(ConfigInfo)],

@@ -66,6 +66,7 @@ struct Options {
     int attention_single_below = 512;  // ... and merging in the kernel: sequences up to this length are not shared at all
     int fused_small = -1;       // fused 3-bit any-precision launches with both roles in the GEMV's own smaller workgroups:
                                 // -1 = when those have 5..8 waves (measured faster there), 1 = whenever they have <= 8, 0 = never
+    int dec_force_cg = 0, dec_force_sg = 0;  // DEC launch plans: chunk groups / segment groups fixed by hand (tuning; 0 = planned)
     int dec_max_chunk_groups = 0;  // DEC launch plans: at most this many chunk groups (atomic adds per output); 0 = the built-in bound
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
@@ -95,6 +96,8 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "attention_single_below")) return &g_opt.attention_single_below;
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     if (!strcmp(name, "dec_max_chunk_groups")) return &g_opt.dec_max_chunk_groups;
+    if (!strcmp(name, "dec_force_cg")) return &g_opt.dec_force_cg;
+    if (!strcmp(name, "dec_force_sg")) return &g_opt.dec_force_sg;
     return nullptr;
 }
 
@@ -258,7 +261,7 @@ constexpr uint32_t kMaxChunkGroups = 4;
 
 // Split the DEC work of one layer over at most `budget` workgroups of `nw` waves: cg chunk groups x sg
 // segment groups, cg <= kMaxChunkGroups (option dec_max_chunk_groups can lower it), minimising the longest
-// per-workgroup path; ties prefer fewer chunk groups.  The row list of a workgroup must fit in LDS: only a
+// per-workgroup path.  The row list of a workgroup must fit in LDS: only a
 // row list that fits with no allowed cg (k_chunk in the hundreds at K > 16384) lifts the bound.
 int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t nw, DecPlan* pl) {
     const uint32_t num_chunks = cdiv(K, 1024);
@@ -273,8 +276,10 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t
     for (int pass = 0; pass < 2 && best_cg == 0; ++pass) {
         const uint32_t cg_max = pass == 0 ? std::min(num_chunks, cap) : num_chunks;
         for (uint32_t cg = 1; cg <= cg_max; ++cg) {
+            if (g_opt.dec_force_cg > 0 && pass == 0 && cg != std::min((uint32_t)g_opt.dec_force_cg, cg_max)) continue;
             const uint32_t sg_max = std::min(nseg, std::max(1u, budget / cg));
             for (uint32_t sg = 1; sg <= sg_max; ++sg) {
+                if (g_opt.dec_force_sg > 0 && pass == 0 && sg != std::min((uint32_t)g_opt.dec_force_sg, sg_max)) continue;
                 const uint32_t cpb = cdiv(num_chunks, cg), spb = cdiv(nseg, sg);
                 const uint32_t slots = (cpb * std::max(k_chunk, 1u) + 1u) & ~1u;   // even: keeps the LDS arrays behind the row list 16-byte aligned
                 const size_t lds = dec_lds_bytes(slots, nw);
@@ -284,7 +289,11 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t
                 // workgroup budget is a last resort
                 const uint32_t sb = std::min(spb, nw), rl = nw / sb;
                 const uint64_t batches = (uint64_t)cdiv(spb, nw) * cdiv(slots, rl * 8);
-                const uint64_t cost = batches * 1000 + (uint64_t)cdiv(cpb, teams) * 600 + (uint64_t)cg * 10 +
+                // Ties go to MORE chunk groups (within the bound): a workgroup then reads wider pieces of fewer rows, and
+                // pieces of one row are contiguous in host memory.  Measured, DEC alone at k_chunk 32 with the same
+                // number of batches: 4096 x 4096 15.3 us with 1 chunk group x 8 segment groups, 12.3 us with 4 x 2 or
+                // 4 x 8; 14336 x 4096 41.6 / 32.0 / 26.3 us with 1 / 2 / 4 chunk groups; 28672 x 8192 108 / 88 / 79 us.
+                const uint64_t cost = batches * 1000 + (uint64_t)cdiv(cpb, teams) * 600 + (uint64_t)(64u - std::min(cg, 64u)) * 10 +
                                       (cg * sg > budget ? 500000ull : 0);
                 if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
             }
@@ -614,6 +623,18 @@ int decdec_debug_read_trace(uint64_t* out, int workgroups) {
     DD_HIP(hipDeviceSynchronize());
     DD_HIP(hipMemcpy(out, g_trace_dev, sizeof(uint64_t) * 8 * (size_t)workgroups, hipMemcpyDeviceToHost));
     DD_HIP(hipMemset(g_trace_dev, 0, sizeof(uint64_t) * 8 * kTraceBlocks));
+    return kOk;
+}
+
+int decdec_debug_read_probe(const void* src, uint64_t row_bytes, uint64_t rows, uint32_t vec_words, uint32_t blocks,
+                            int scramble, void* sink, void* stream) {
+    DD_CHECK(src && sink, "null pointer argument");
+    DD_CHECK(vec_words == 1 || vec_words == 2 || vec_words == 4, "vec_words must be 1, 2 or 4");
+    DD_CHECK(rows >= 1 && blocks >= 1, "rows and blocks must be positive");
+    DD_CHECK(row_bytes >= 256ull * vec_words && row_bytes % (256ull * vec_words) == 0,
+             "row_bytes must be a positive multiple of 256 * vec_words");
+    DD_CHECK(((uintptr_t)src % 16) == 0, "src must be 16-byte aligned");
+    DD_HIP(launch_read_probe(src, row_bytes, rows, vec_words, blocks, scramble, sink, (hipStream_t)stream));
     return kOk;
 }
 
@@ -960,6 +981,69 @@ int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* 
     if (!have_dec && g_opt.fusion) { DD_HIP(launch_anyprec(dtype, bits, pl.p, pl.d, s)); return kOk; }
     return two_stream(c, &dp, have_dec, dtype, s,
                       [&](hipStream_t sub) { return launch_anyprec(dtype, bits, pl.p, pl.d, sub); });
+}
+
+// Several any-precision layers that read the same input, in one launch (q | k | v, gate | up).  A layer whose config
+// handle is 0, or whose config has k_chunk 0, runs its base GEMV only.
+int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                             const void* const* qweights, const void* const* luts, int bits, int dtype, uint32_t K,
+                             const uint32_t* out_features, void* stream) {
+    DD_CHECK(n >= 1 && n <= (uint32_t)kMaxBatch, "a batch holds 1 to %d layers, got %u", kMaxBatch, n);
+    DD_CHECK(outputs && qweights && luts && out_features, "null pointer argument");
+    DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
+    for (uint32_t i = 0; i < n; ++i)
+        for (uint32_t j = 0; j < i; ++j)
+            DD_CHECK(outputs[i] != outputs[j], "the layers of a batch must have distinct outputs");
+    if (!g_opt.fusion || (bits != 3 && bits != 4)) {
+        // no batched kernel for this case: one call per layer, same result
+        for (uint32_t i = 0; i < n; ++i) {
+            const int rc = (configs && configs[i])
+                ? decdec_dec_anyprec(configs[i], input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], stream)
+                : decdec_anyprec_gemv(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], stream);
+            if (rc != kOk) return rc;
+        }
+        return kOk;
+    }
+    BatchParams<AnyprecParams> b;
+    memset(&b, 0, sizeof(b));
+    b.n = n;
+    LaunchDims d{0, 1024u, 0};
+    uint32_t dec_total = 0, gemv_total = 0;
+    double dec_us = 0.0, weight_bytes = 0.0;
+    bool any_dec = false;
+    for (uint32_t i = 0; i < n; ++i) {
+        Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
+        bool have_dec = false;
+        if (configs && configs[i]) {
+            int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
+            if (rc != kOk) return rc;
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i]) == 0;
+            b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
+        }
+        AnyprecPlan pl;
+        int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], true, &pl);
+        if (rc != kOk) return rc;
+        b.gp[i] = pl.p;
+        d.lds = std::max(d.lds, pl.d.lds);
+        if (have_dec) {
+            dec_total += c->plans[2].cg * c->plans[2].sg;
+            d.lds = std::max(d.lds, c->plans[2].lds);
+            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
+            any_dec = true;
+        }
+        gemv_total += pl.d.grid;
+        weight_bytes += (double)bits * out_features[i] * K / 8.0;
+        b.dec_end[i] = dec_total;
+        b.gemv_end[i] = gemv_total;
+    }
+    for (uint32_t i = n; i < (uint32_t)kMaxBatch; ++i) { b.dec_end[i] = dec_total; b.gemv_end[i] = gemv_total; }
+    d.grid = dec_total + gemv_total;
+    // two workgroups per compute unit while the DEC roles together (one latency floor, the bytes of all layers) are
+    // not the longer part by a margin -- the single-layer rule applied to the batch
+    if (g_opt.fused_two_per_cu >= 0) d.two_per_cu = g_opt.fused_two_per_cu != 0;
+    else d.two_per_cu = !any_dec || (8.0 + dec_us) < 0.9 * gemv_estimate_us(kAnyprec, weight_bytes);
+    DD_HIP(launch_dec_anyprec_batch(dtype, bits, b, d, (hipStream_t)stream));
+    return kOk;
 }
 
 int decdec_dec_lutgemm(uint64_t h, const void* input, void* output, const void* qw, const void* alpha,

@@ -18,6 +18,22 @@ __global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_anyprec_kernel(co
     else anyprec_role<DT, BITS>(gp, blockIdx.x - dec_blocks, smem);
 }
 
+// Up to kMaxBatch layers on one input in one launch: a workgroup finds its layer and plays the DEC or the GEMV role
+// for it, exactly as in the single-layer kernel above.
+template <int DT, int BITS, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_anyprec_batch_kernel(const BatchParams<AnyprecParams> b) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t ndec = b.dec_end[kMaxBatch - 1];
+    uint32_t layer, local;
+    if (blockIdx.x < ndec) {
+        batch_locate(b.dec_end, blockIdx.x, layer, local);
+        dec_role<DT>(b.dp[layer], local, smem);
+    } else {
+        batch_locate(b.gemv_end, blockIdx.x - ndec, layer, local);
+        anyprec_role<DT, BITS>(b.gp[layer], local, smem);
+    }
+}
+
 // The same two roles in workgroups of NW (4 or 8) waves, eight waves per SIMD: the GEMV role runs in workgroups of
 // its standalone size, and a DEC workgroup holds an eighth or a quarter of a compute unit.
 template <int DT, int NW>
@@ -100,6 +116,22 @@ hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t de
         DD_BITS_SWITCH(bits, hipLaunchKernelGGL((dec_anyprec_kernel<kBF16, B, false>), grid, block, d.lds, s, dp, dec_blocks, gp));
     } else {
         return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_anyprec_batch(int dt, int bits, const BatchParams<AnyprecParams>& b, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(d.grid), block(d.block);
+    if ((dt != kFP16 && dt != kBF16) || (bits != 3 && bits != 4) || d.block != 1024u) return hipErrorInvalidValue;
+    if (bits == 3 && d.two_per_cu) {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_anyprec_batch_kernel<kFP16, 3, true>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_anyprec_batch_kernel<kBF16, 3, true>), grid, block, d.lds, s, b);
+    } else if (bits == 3) {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_anyprec_batch_kernel<kFP16, 3, false>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_anyprec_batch_kernel<kBF16, 3, false>), grid, block, d.lds, s, b);
+    } else {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_anyprec_batch_kernel<kFP16, 4, false>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_anyprec_batch_kernel<kBF16, 4, false>), grid, block, d.lds, s, b);
     }
     return hipGetLastError();
 }

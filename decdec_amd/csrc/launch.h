@@ -22,6 +22,26 @@ struct LaunchDims {
 // DEC is the longer role use the unconstrained instance, one workgroup per unit.
 #define DD_TWO_PER_CU(on) __attribute__((amdgpu_waves_per_eu((on) ? 8 : 4, 8)))
 
+// Several layers that read the same activation vector in ONE launch (q | k | v, gate | up): the DEC workgroups of all
+// layers come first in the grid (their host-memory reads start at once), then the GEMV workgroups, layer by layer.
+// dec_end / gemv_end are running totals of workgroups over the layers (entries past n repeat the last total).
+constexpr int kMaxBatch = 4;
+template <typename GemvParams>
+struct BatchParams {
+    uint32_t n;
+    uint32_t dec_end[kMaxBatch];
+    uint32_t gemv_end[kMaxBatch];
+    DecParams dp[kMaxBatch];
+    GemvParams gp[kMaxBatch];
+};
+// the layer a workgroup of a batch belongs to, and its index inside that layer's share of the grid
+__device__ __forceinline__ void batch_locate(const uint32_t (&end)[kMaxBatch], uint32_t id, uint32_t& layer, uint32_t& local) {
+    layer = 0; local = id;
+#pragma unroll
+    for (int j = 0; j + 1 < kMaxBatch; ++j)
+        if (id >= end[j]) { layer = (uint32_t)j + 1u; local = id - end[j]; }
+}
+
 // Standalone kernels.
 hipError_t launch_dec(int dt, const DecParams& p, const LaunchDims& d, hipStream_t s);
 hipError_t launch_anyprec(int dt, int bits, const AnyprecParams& p, const LaunchDims& d, hipStream_t s);
@@ -30,11 +50,16 @@ hipError_t launch_anyprec_dequant(int dt, int bits, const uint32_t* qweight, con
 hipError_t launch_lutgemm(int dt, const LutgemmParams& p, const LaunchDims& d, hipStream_t s);
 hipError_t launch_sqllm(int dt, const SqllmParams& p, const LaunchDims& d, hipStream_t s);
 hipError_t launch_burner(uint32_t blocks, long long iters, hipStream_t s);
+hipError_t launch_read_probe(const void* src, unsigned long long row_bytes, unsigned long long rows, uint32_t vec_words,
+                             uint32_t blocks, int scramble, void* sink, hipStream_t s);
 
 // Single-launch fused kernels: workgroups [0, dec_blocks) play the DEC role, the rest the base GEMV.
 // d.grid counts the GEMV workgroups only; d.block is 1024.
 hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t dec_blocks,
                               const AnyprecParams& gp, const LaunchDims& d, hipStream_t s);
+// A batch of up to kMaxBatch any-precision layers on one input, each with or without DEC (3 or 4 bits; d.grid and
+// d.lds cover all layers; d.block is 1024).
+hipError_t launch_dec_anyprec_batch(int dt, int bits, const BatchParams<AnyprecParams>& b, const LaunchDims& d, hipStream_t s);
 // 3-bit, both roles in workgroups of `nw` (4 or 8) waves = d.block / 64; dp carries the DEC plan for that size.
 hipError_t launch_dec_anyprec_small(int dt, uint32_t nw, const DecParams& dp, uint32_t dec_blocks,
                                     const AnyprecParams& gp, const LaunchDims& d, hipStream_t s);

@@ -19,6 +19,9 @@ _DT_NAME = {torch.float32: "FP32", torch.float16: "FP16", torch.bfloat16: "BF16"
 # config handle -> tensors whose storage the config borrows (thresholds) -- the reference leaves
 # keeping them alive to the caller; holding a reference here costs nothing and removes a hazard
 _KEEPALIVE: dict[int, tuple] = {}
+# context handle -> the two scratch tensors the context borrows (same reasoning: a context whose buffers were
+# garbage-collected would let DEC write its selection into whatever the allocator put there next)
+_CONTEXT_KEEPALIVE: dict[int, tuple] = {}
 _CONFIG_DTYPE: dict[int, torch.dtype] = {}
 _CONFIG_SHAPE: dict[int, tuple[int, int]] = {}
 
@@ -60,12 +63,14 @@ def create_dec_context(num_tb: int, selected_rows_buffer: torch.Tensor,
     _lib.check(_lib.load().decdec_create_dec_context(
         int(num_tb), dt, selected_activations_buffer.numel(), _ptr(selected_rows_buffer),
         _ptr(selected_activations_buffer), ctypes.byref(handle)))
+    _CONTEXT_KEEPALIVE[int(handle.value)] = (selected_rows_buffer, selected_activations_buffer)
     return int(handle.value)
 
 
 def destroy_dec_context(dec_context: int) -> None:
     """Not in the reference (which leaks contexts); releases the sub-stream and event."""
     _lib.check(_lib.load().decdec_destroy_dec_context(int(dec_context)))
+    _CONTEXT_KEEPALIVE.pop(int(dec_context), None)
 
 
 def create_dec_config(dec_context: int, k_chunk: int, q_residual: torch.Tensor,
@@ -315,6 +320,28 @@ def dec_anyprec(dec_config: int, input, output, q_weight, lut, bitwidth: int) ->
                                               int(bitwidth), _dt(input), input.size(2), output.size(2), _stream()))
 
 
+def dec_anyprec_batch(dec_configs, input, outputs, q_weights, luts, bitwidth: int) -> None:
+    """Layers that read the same `input`, in one launch: layer i is dec_anyprec(dec_configs[i], input, outputs[i],
+    q_weights[i], luts[i], bitwidth), or anyprec_gemv when dec_configs[i] is 0 / None (dec_configs may be None).
+    Not in the reference (which concatenates such projections' weights instead)."""
+    n = len(outputs)
+    _check(1 <= n <= 4 and len(q_weights) == n and len(luts) == n, "a batch holds 1 to 4 layers")
+    cfgs = [int(c) if c else 0 for c in (dec_configs if dec_configs is not None else [0] * n)]
+    _check(len(cfgs) == n, "one config (or 0) per layer")
+    _check(input.dtype in (torch.float16, torch.bfloat16), "Unsupported data type.")
+    for c, out, qw, lut in zip(cfgs, outputs, q_weights, luts):
+        if c:
+            _check_dec_io(c, input, out)
+        _check_anyprec(input, out, qw, lut, bitwidth)
+    arr_c = (ctypes.c_uint64 * n)(*cfgs)
+    arr_o = (ctypes.c_void_p * n)(*[_ptr(t) for t in outputs])
+    arr_q = (ctypes.c_void_p * n)(*[_ptr(t) for t in q_weights])
+    arr_l = (ctypes.c_void_p * n)(*[_ptr(t) for t in luts])
+    arr_n = (ctypes.c_uint32 * n)(*[t.size(2) for t in outputs])
+    _lib.check(_lib.load().decdec_dec_anyprec_batch(n, arr_c, _ptr(input), arr_o, arr_q, arr_l, int(bitwidth), _dt(input),
+                                                    input.size(2), arr_n, _stream()))
+
+
 def dec_lutgemm(dec_config: int, input, output, q_weight, alpha, q_bias, bitwidth: int, group_size: int) -> None:
     """decdec.cu:701-721."""
     _check(input.dtype in _DT, "Unsupported data type.")
@@ -368,4 +395,4 @@ REFERENCE_API = (
     "dec", "unfused_dec", "anyprec_dequant", "anyprec_gemv", "lutgemm_gemv", "sqllm_gemv",
     "dec_anyprec", "dec_lutgemm", "dec_sqllm", "dummy_anyprec", "dummy_lutgemm", "dummy_sqllm",
 )
-__all__ = list(REFERENCE_API) + ["destroy_dec_context"]
+__all__ = list(REFERENCE_API) + ["destroy_dec_context", "dec_anyprec_batch"]

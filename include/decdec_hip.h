@@ -65,7 +65,8 @@ int decdec_version(void);
  * workgroup per head, which is faster there; default 512, 0 = always share),
  * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows),
  * "dec_max_chunk_groups" (DEC launch plans made from now on use at most this many chunk groups, i.e. atomic adds per
- * output: 1 to 4; 0 = the built-in bound of 4 [default]), "dec_trace" (see
+ * output: 1 to 4; 0 = the built-in bound of 4 [default]), "dec_force_cg" / "dec_force_sg" (DEC launch plans made from
+ * now on use this many chunk groups / segment groups where the shape allows; tuning aid, 0 = planned [default]), "dec_trace" (see
  * decdec_debug_read_trace).  No counterpart in the reference. */
 int decdec_set_option(const char* name, int value);
 int decdec_get_option(const char* name, int* value);
@@ -153,6 +154,19 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
                        int bitwidth, int dtype, uint32_t in_features, uint32_t out_features,
                        int dummy_cu, int64_t dummy_iters, void* stream);
 
+/* Several any-precision layers that read the SAME input vector, in one launch: q | k | v and gate | up of a decoder
+ * layer are independent given their input, and one launch pays the launch and selection latencies once instead of once
+ * per layer.  Layer i: config configs[i] (0, or a config with k_chunk 0: base GEMV only; configs may be NULL when no
+ * layer has DEC), output outputs[i] (out_features[i] elements, distinct per layer, zeroed by the caller as for the
+ * single-layer ops), qweights[i], luts[i].  1 to 4 layers, the same bitwidth and dtype; results are those of n
+ * decdec_dec_anyprec / decdec_anyprec_gemv calls.  Configs of one batch that belong to the same context write their
+ * selections into the same scratch buffers at the same time: give each layer of a batch a context of its own if the
+ * selection is read back.  No counterpart in the reference, which fuses such projections by concatenating their
+ * weights (end-to-end/model.py wqkv, w1w3). */
+int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                             const void* const* qweights, const void* const* luts, int bitwidth, int dtype,
+                             uint32_t in_features, const uint32_t* out_features, void* stream);
+
 /* Decode-step helpers for a caller that drives the linear layers from a captured decode step (the
  * reference leaves these operations to torch.compile, end-to-end/generate.py; they have no counterpart in
  * its extension).  All tensors are fp16 or bf16 in device memory; `pos_device` points at the token position
@@ -225,6 +239,14 @@ int decdec_greedy_pick(const void* logits, uint32_t n, int dtype, void* workspac
  * library-owned device buffer; this copies the first `workgroups` x 8 stamps to the host (it
  * synchronises the device).  No counterpart in the reference. */
 int decdec_debug_read_trace(uint64_t* stamps_out, int workgroups);
+/* Diagnostics: a plain read kernel, nothing but loads -- the rate a fetch can reach on the memory `src` points at
+ * (pinned host memory through its device address: the ceiling of the zero-copy residual fetch over the host link;
+ * device memory: the ceiling of a streaming read).  Reads `rows` rows of `row_bytes` bytes (a multiple of
+ * 256 * vec_words) laid out back to back, with `blocks` workgroups of 1024 threads, vec_words (1, 2, 4) dwords per lane
+ * and request, eight requests in flight per wave; `scramble` != 0 visits the rows in a scattered order, as DEC's
+ * selected rows are.  `sink`: 4 bytes of device memory.  No counterpart in the reference. */
+int decdec_debug_read_probe(const void* src, uint64_t row_bytes, uint64_t rows, uint32_t vec_words,
+                            uint32_t blocks, int scramble, void* sink, void* stream);
 
 /* Host-only helpers (no GPU needed).  decdec_bucket_floors evaluates the selector's 32 bucket
  * floors exactly as dec.cu:117-130 does, in `dtype` arithmetic; decdec_reference_geometry evaluates

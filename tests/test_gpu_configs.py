@@ -224,6 +224,54 @@ def test_unfused_dec_with_magnitude_sorted_indices(K, N, k_chunk, waves, c_oracl
     ext.destroy_dec_config(cfg)
 
 
+@pytest.mark.parametrize("dt,bits", [("fp16", 3), ("bf16", 3), ("fp16", 4), ("fp16", 5)])
+def test_batched_layers_match_the_oracle_layer_by_layer(dt, bits, c_oracle):
+    """dec_anyprec_batch: q | k | v of a Llama-3-8B layer (one input, three outputs) in one launch, every layer with
+    its own config and context; then the same batch with DEC on the middle layer only, and without any config.
+    Each output against the oracle, each context's selection bit-exact.  (5 bits: the per-layer fallback.)"""
+    from tests.helpers import TORCH_DT
+    dtype = TORCH_DT[dt]
+    K, Ns, k_chunk = 4096, (4096, 1024, 1032), 32
+    g = torch.Generator().manual_seed(7)
+    x = F.make_activation(K, g, dtype=dtype)
+    xn = np_of(x)
+    layers = []
+    for li, N in enumerate(Ns):
+        W = (torch.randn(N, K, generator=g) * 0.02).half()
+        idx, lut = F.quantize_uniform_rows(W, bits)
+        cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32)
+        scales = (torch.rand(N, generator=g) * 1e-3 + 5e-4).to(dtype)
+        th = F.calibrate_thresholds(K, g, draws=8, dtype=dtype)
+        ctx, rows, acts = _ctx(16, K, dtype)
+        cfg = ext.create_dec_config(ctx, k_chunk, cheat, scales, th)
+        qweight = F.pack_anyprec(idx, bits)
+        layers.append(dict(N=N, qweight=qweight, lut=lut.to(dtype), cheat=cheat, scales=scales, th=th, cfg=cfg, rows=rows, acts=acts,
+                           base=c_oracle.anyprec_gemv(xn, qweight.numpy(), np_of(lut.to(dtype)), bits, dt)))
+    qws = [l["qweight"].cuda() for l in layers]
+    luts = [l["lut"].cuda() for l in layers]
+    xc = x.cuda()
+    for mode in ("all", "middle", "none"):
+        outs = [torch.zeros(1, 1, l["N"], dtype=dtype, device="cuda") for l in layers]
+        for l in layers:
+            l["rows"].fill_(-7)
+        cfgs = {"all": [l["cfg"] for l in layers], "middle": [0, layers[1]["cfg"], None], "none": None}[mode]
+        ext.dec_anyprec_batch(cfgs, xc, outs, qws, luts, bits)
+        torch.cuda.synchronize()
+        for li, l in enumerate(layers):
+            with_dec = cfgs is not None and bool(cfgs[li])
+            want = l["base"]
+            if with_dec:
+                want_rows, _, _ = O.select_channels(xn, np_of(l["th"]), k_chunk, dt)
+                k = k_chunk * K // 1024
+                assert np.array_equal(l["rows"].cpu().numpy()[:k], want_rows[:k]), (mode, li)
+                want = want + c_oracle.dec_apply(xn, l["cheat"].numpy(), np_of(l["scales"]), want_rows[:k], dt)
+            else:
+                assert (l["rows"].cpu().numpy() == -7).all(), (mode, li)
+            check_output(np_of(outs[li]).reshape(-1), want, dt, (mode, li, bits))
+    for l in layers:
+        ext.destroy_dec_config(l["cfg"])
+
+
 # --------------------------------------------------------------------------------------------------
 # Phi-3-medium: LUT-GEMM 3-bit, group 128, with DEC
 # --------------------------------------------------------------------------------------------------
