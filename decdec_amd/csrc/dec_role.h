@@ -298,7 +298,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             for (int s = 0; s < 4; ++s) {
                 if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
             }
-            if (ttid == 0) hdr[1] = total;
+            if (ttid == 0) { hdr[1] = total; hdr[2] = dec_attempt_bucket_rt(us); }
         }
         if (ttid == 0) hdr[0] = fast ? kTeamFast : kTeamGeneral;
     } else if (ttid == 0) {
@@ -314,39 +314,38 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
         any_general = any_general || h[0] == kTeamGeneral;
         any_big = any_big || (h[0] == kTeamFast && h[1] > (uint32_t)kWave);
     }
-    const u32x2 hd = *(const u32x2*)hdr;
+    const u32x4 hd = *(const u32x4*)hdr;                    // state, candidates, bucket of the winning cut-off
     const bool fast = hd[0] == kTeamFast;
     const uint32_t total = hd[1];
     dec_stamp(p, blockIdx.x, 6);
     if (fast && total <= (uint32_t)kWave) {
-        // The usual case: at most 64 candidates.  One wave holds a candidate per lane and ranks them all-pairs
-        // against the key list read back as broadcasts; nothing here needs a workgroup barrier.
+        // The usual case: at most 64 candidates, in channel order.  One wave holds a candidate per lane and ranks
+        // them by (bucket, channel) with ballots only: a candidate's position is the number of candidates in lower
+        // buckets plus the number of earlier lanes in its own bucket.  Nothing here needs a workgroup barrier or a
+        // trip through LDS beyond reading the candidate itself.
         if (tw == 0) {
-            uint32_t mykey = 0xFFFFFFFFu;                  // padding: never smaller than a real key
-            float xs = 0.f;
-            if (lane < total) {
-                xs = cx[lane];
-                const float ca = __builtin_fabsf(xs);
-                uint32_t bkt = 0;
+            const bool valid = lane < total;
+            const float xs = valid ? cx[lane] : 0.f;
+            const uint32_t chl = valid ? key[lane] : 0u;
+            const float ca = __builtin_fabsf(xs);
+            // bucket = number of floors above the candidate; candidates lie at or above the winning cut-off
+            // floor[hd[2]], so later (smaller) floors cannot be above them
+            const uint32_t nfl = hd[2] + 1u;                   // uniform
+            uint32_t bkt = 0;
+#pragma unroll 4
+            for (uint32_t i = 0; i < nfl; ++i) bkt += (ca < dec_floor(myfloor, (int)i)) ? 1u : 0u;
+            unsigned long long eq = total >= 64u ? ~0ull : ((1ull << total) - 1ull);    // lanes whose bucket equals mine
+            unsigned long long lt = 0ull;                                               // lanes whose bucket is lower
 #pragma unroll
-                for (int i = 0; i < kBuckets; ++i) bkt += (ca < dec_floor(myfloor, i)) ? 1u : 0u;
-                mykey = (bkt << 10) | key[lane];
+            for (int k = 4; k >= 0; --k) {
+                const bool mybit = ((bkt >> k) & 1u) != 0u;
+                const unsigned long long bk = __ballot(valid && mybit);
+                lt |= mybit ? (eq & ~bk) : 0ull;
+                eq &= mybit ? bk : ~bk;
             }
-            key[lane] = mykey;
-            uint32_t pos = 0;
-            const u32x4* kp = (const u32x4*)key;
-            // 32 keys per step, all reads of a step in flight together (the padding keys count nothing)
-#pragma unroll 1
-            for (uint32_t h = 0; h * 32u < total; ++h) {
-                u32x4 k4[8];
-#pragma unroll
-                for (int v = 0; v < 8; ++v) k4[v] = kp[h * 8u + v];
-#pragma unroll
-                for (int v = 0; v < 8; ++v)
-                    pos += (k4[v][0] < mykey) + (k4[v][1] < mykey) + (k4[v][2] < mykey) + (k4[v][3] < mykey);
-            }
-            if (lane < total && pos < kc) {
-                const uint32_t ch = lo + (mykey & 1023u);
+            const uint32_t pos = (uint32_t)__popcll(lt) + ballot_rank(eq);
+            if (valid && pos < kc) {
+                const uint32_t ch = lo + chl;
                 const uint32_t slot = t_local * p.k_chunk + pos;
                 lrows[slot] = (int32_t)ch;
                 lacts[slot] = xs;
