@@ -184,12 +184,15 @@ constexpr int kTeamWords = 32 + 2 * kMaxCand + 8;
 constexpr size_t kTeamBytes = (size_t)kTeamWords * 4 + (size_t)16 * kMaxCand;
 enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u };
 
+// The cut-offs tried: every bucket just below the calibrated threshold (floor[15] = thresholds[k - 1]: with
+// activations like the calibration set about kc channels lie above it, and one bucket further down adds about
+// kc / 2 more, so the first window that holds kc channels rarely holds more than 64), coarser further down.
 __device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) {
-    return u == 0 ? 15u : u == 1 ? 18u : u == 2 ? 21u : u == 3 ? 23u : u == 4 ? 25u : u == 5 ? 27u : u == 6 ? 29u : 31u;
+    return u == 0 ? 15u : u == 1 ? 16u : u == 2 ? 17u : u == 3 ? 18u : u == 4 ? 20u : u == 5 ? 23u : u == 6 ? 27u : 31u;
 }
 // the same for a wave-uniform run-time attempt number: one byte per attempt
 __device__ __forceinline__ uint32_t dec_attempt_bucket_rt(uint32_t u) {
-    const unsigned long long tab = 0x1F1D1B191715120Full;   // bytes 15, 18, 21, 23, 25, 27, 29, 31
+    const unsigned long long tab = 0x1F1B17141211100Full;   // bytes 15, 16, 17, 18, 20, 23, 27, 31
     return (uint32_t)(tab >> (8u * u)) & 0xFFu;
 }
 
@@ -322,8 +325,10 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
         // The usual case: at most 64 candidates, in channel order.  One wave holds a candidate per lane and ranks
         // them by (bucket, channel) with ballots only: a candidate's position is the number of candidates in lower
         // buckets plus the number of earlier lanes in its own bucket.  Nothing here needs a workgroup barrier or a
-        // trip through LDS beyond reading the candidate itself.
-        if (tw == 0) {
+        // trip through LDS beyond reading the candidate itself.  Team j ranks on its wave j: waves w and w + 4 of a
+        // workgroup share a SIMD, so the ranking waves of the four teams sit on four different SIMDs (a single
+        // wave issues an instruction every four cycles at best; four ranking waves on one SIMD took 2.2x as long).
+        if (tw == (team & (uint32_t)(kSelWaves - 1))) {
             const bool valid = lane < total;
             const float xs = valid ? cx[lane] : 0.f;
             const uint32_t chl = valid ? key[lane] : 0u;
@@ -332,7 +337,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             // floor[hd[2]], so later (smaller) floors cannot be above them
             const uint32_t nfl = hd[2] + 1u;                   // uniform
             uint32_t bkt = 0;
-#pragma unroll 4
+#pragma unroll 1
             for (uint32_t i = 0; i < nfl; ++i) bkt += (ca < dec_floor(myfloor, (int)i)) ? 1u : 0u;
             unsigned long long eq = total >= 64u ? ~0ull : ((1ull << total) - 1ull);    // lanes whose bucket equals mine
             unsigned long long lt = 0ull;                                               // lanes whose bucket is lower
