@@ -266,7 +266,7 @@ constexpr uint32_t kMaxChunkGroups = 4;
 int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t nw, DecPlan* pl) {
     const uint32_t num_chunks = cdiv(K, 1024);
     const uint32_t nseg = cdiv(M, 64);
-    const uint32_t teams = std::max(1u, nw / 4u);
+    const uint32_t teams = nw >= 16u ? 4u : std::max(1u, nw / 2u);     // chunks a workgroup selects at a time (dec_role.h, DecTeam)
     budget = std::max(1u, budget);
     uint32_t cap = kMaxChunkGroups;
     if (g_opt.dec_max_chunk_groups >= 1) cap = std::min(cap, (uint32_t)g_opt.dec_max_chunk_groups);

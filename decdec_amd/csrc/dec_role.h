@@ -52,11 +52,11 @@ constexpr int kMinDecWaves = 4;                              // smallest: the fo
 constexpr int kMaxCand = 256;                                // fast-path candidate list capacity
 constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per thread and segment batch
 
+__host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves);
 __host__ __device__ inline size_t dec_lds_bytes(uint32_t slots, uint32_t nwaves = kDecWaves) {
     // row list (index + activation) + counters/prefix of the general selection + the buffer shared by the
-    // cross-wave reduction ([nwaves][8][64] floats) and the selection teams (one area per four waves)
-    const size_t red = (size_t)nwaves * 8 * kWave * 4;
-    const size_t teams = (size_t)(nwaves / 4) * ((size_t)(32 + 2 * kMaxCand + 8) * 4 + (size_t)16 * kMaxCand);
+    // cross-wave reduction ([nwaves][8][64] floats) and the selection teams
+    const size_t red = (size_t)nwaves * 8 * kWave * 4, teams = dec_team_lds_bytes(nwaves);
     return (size_t)slots * 8 + 2 * 512 * 4 + (red > teams ? red : teams);
 }
 
@@ -176,12 +176,26 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // chunk only.  A chunk the fast path cannot take (non-monotone floors, more than kMaxCand candidates,
 // k_chunk > kMaxCand) is afterwards selected by the whole workgroup on the general path.
 constexpr int kAttempts = 8;
-constexpr int kSelWaves = 4;                                 // waves of a team
-constexpr int kTeamThreads = kSelWaves * kWave;
-// per-team LDS: candidate counts [kAttempts][kSelWaves], keys [kMaxCand], activations [kMaxCand], header
-// (state, candidate count; padded), partial ranks [16][kMaxCand] bytes
-constexpr int kTeamWords = 32 + 2 * kMaxCand + 8;
-constexpr size_t kTeamBytes = (size_t)kTeamWords * 4 + (size_t)16 * kMaxCand;
+// Team geometry by workgroup size.  A 16-wave workgroup has four teams of four waves (four channels per lane, up to
+// 256 candidates per chunk on the fast path); smaller workgroups have teams of two waves (eight channels per lane,
+// up to 128 candidates): an 8-wave workgroup then still selects four chunks at a time, a 4-wave one two.
+template <int NW> struct DecTeam {
+    static constexpr int kWaves = NW >= 16 ? 4 : 2;                 // waves of a team
+    static constexpr int kThreads = kWaves * kWave;
+    static constexpr int kTeams = NW / kWaves;
+    static constexpr int kLaneChannels = kChunk / kThreads;        // channels a scanning lane owns: 4 or 8
+    static constexpr int kCand = NW >= 16 ? kMaxCand : kMaxCand / 2;   // fast-path candidate capacity: one per team thread
+    // per-team LDS: candidate counts [kAttempts][4], keys [kCand], activations [kCand], header (state, candidate
+    // count, bucket of the winning cut-off; padded), partial ranks [kCand / 16][kCand] bytes
+    static constexpr int kWords = 32 + 2 * kCand + 8;
+    static constexpr int kHdrWord = 32 + 2 * kCand;
+    static constexpr size_t kBytes = (size_t)kWords * 4 + (size_t)(kCand / 16) * kCand;
+};
+__host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves) {
+    return nwaves >= 16 ? (size_t)DecTeam<16>::kTeams * DecTeam<16>::kBytes
+                        : (nwaves >= 8 ? (size_t)DecTeam<8>::kTeams * DecTeam<8>::kBytes
+                                       : (size_t)DecTeam<4>::kTeams * DecTeam<4>::kBytes);
+}
 enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u };
 
 // The cut-offs tried: every bucket just below the calibrated threshold (floor[15] = thresholds[k - 1]: with
@@ -196,13 +210,13 @@ __device__ __forceinline__ uint32_t dec_attempt_bucket_rt(uint32_t u) {
     return (uint32_t)(tab >> (8u * u)) & 0xFFu;
 }
 
-// The four activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
+// The activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
 // costs a branch and a full wait each).
 // Storage bits only: converting at once would make the lane wait for the loads where they are issued.
-template <int DT>
-__device__ __forceinline__ void dec_load_x4(const DecParams& p, uint32_t lo, uint32_t len, uint32_t ch0, uint32_t (&xr)[4]) {
+template <int DT, int C>
+__device__ __forceinline__ void dec_load_x(const DecParams& p, uint32_t lo, uint32_t len, uint32_t ch0, uint32_t (&xr)[C]) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) xr[s] = Elem<DT>::load_raw(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
+    for (int s = 0; s < C; ++s) xr[s] = Elem<DT>::load_raw(p.x, lo + ((ch0 + s < len) ? ch0 + s : len - 1u));
 }
 
 __device__ __forceinline__ uint32_t dec_chunk_len(const DecParams& p, uint32_t c) {
@@ -217,13 +231,17 @@ template <int DT, int NW>
 __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cgid, uint32_t t0, uint32_t nlocal,
                                                  int32_t* lrows, float* lacts, uint32_t* cnt,
                                                  uint32_t* pre, float* red, bool write_global,
-                                                 bool have_xpre, const uint32_t (&xpre)[4], const float myfloor) {
+                                                 bool have_xpre, const uint32_t (&xpre)[DecTeam<NW>::kLaneChannels],
+                                                 const float myfloor) {
     using E = Elem<DT>;
-    constexpr uint32_t kTeams = NW / kSelWaves;
+    using T = DecTeam<NW>;
+    constexpr uint32_t kTeams = T::kTeams, kSelWaves = T::kWaves, kTeamThreads = T::kThreads, kCand = T::kCand;
+    constexpr int C = T::kLaneChannels;
+    constexpr size_t kTeamBytes = T::kBytes;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t team = wave / (uint32_t)kSelWaves, tw = wave % (uint32_t)kSelWaves;
-    const uint32_t ttid = tid & (uint32_t)(kTeamThreads - 1);
+    const uint32_t team = wave / kSelWaves, tw = wave % kSelWaves;
+    const uint32_t ttid = tid & (kTeamThreads - 1u);
     const uint32_t t_local = t0 + team;
     const uint32_t c = cgid + t_local * p.cg;
     const bool has_chunk = t_local < nlocal;                // uniform per wave
@@ -233,72 +251,73 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     const bool active = has_chunk && kc > 0u;
 
     unsigned char* tbase = (unsigned char*)red + (size_t)team * kTeamBytes;
-    uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][kSelWaves] candidate counts
-    uint32_t* key = wc + 32;                               // [kMaxCand]
-    float* cx = (float*)(key + kMaxCand);                  // [kMaxCand]
-    uint32_t* hdr = key + 2 * kMaxCand;                    // state, candidate count
-    uint8_t* pc = tbase + (size_t)kTeamWords * 4;          // [16][kMaxCand] partial ranks (each at most 16)
+    uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][4] candidate counts (kSelWaves used)
+    uint32_t* key = wc + 32;                               // [kCand]
+    float* cx = (float*)(key + kCand);                     // [kCand]
+    uint32_t* hdr = wc + T::kHdrWord;                      // state, candidate count, bucket of the winning cut-off
+    uint8_t* pc = tbase + (size_t)T::kWords * 4;           // [kCand / 16][kCand] partial ranks (each at most 16)
     const bool scanner = active && p.monotone;             // uniform per wave
 
-    // ---- the team scans its chunk: lane l of team wave w owns channels 4 (64 w + l) .. + 3
+    // ---- the team scans its chunk: lane l of team wave w owns channels C (64 w + l) .. + C - 1
     // |x| of the lane's channel s as the selection sees it: NaN, inf and channels past the end are members of no
     // bucket.  Recomputed after the barrier instead of kept: registers held across it are charged to every kernel
     // that contains this role.
-    float xv[4];
-    const uint32_t ch0 = 4u * ttid;
+    float xv[C];
+    const uint32_t ch0 = (uint32_t)C * ttid;
     auto mag = [&](int s) {
         const float v = __builtin_fabsf(xv[s]);
         return (ch0 + (uint32_t)s < len && v < __builtin_inff()) ? v : -__builtin_inff();
     };
     if (scanner) {
-        uint32_t xr[4];
+        uint32_t xr[C];
         if (have_xpre) {                                   // uniform: requested when the workgroup started
 #pragma unroll
-            for (int s = 0; s < 4; ++s) xr[s] = xpre[s];
+            for (int s = 0; s < C; ++s) xr[s] = xpre[s];
         } else {
-            dec_load_x4<DT>(p, lo, len, ch0, xr);
+            dec_load_x<DT, C>(p, lo, len, ch0, xr);
         }
-        asm volatile("" : "+v"(xr[0]), "+v"(xr[1]), "+v"(xr[2]), "+v"(xr[3]));   // first use: here
 #pragma unroll
-        for (int s = 0; s < 4; ++s) xv[s] = E::from_raw(xr[s]);
+        for (int s = 0; s < C; ++s) asm volatile("" : "+v"(xr[s]));             // first use: here
+#pragma unroll
+        for (int s = 0; s < C; ++s) xv[s] = E::from_raw(xr[s]);
         dec_stamp(p, blockIdx.x, 5);
         uint32_t n[kAttempts];
         {
-            float a[4];
+            float a[C];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) a[s] = mag(s);
+            for (int s = 0; s < C; ++s) a[s] = mag(s);
 #pragma unroll
             for (int u = 0; u < kAttempts; ++u) {
                 const float f = dec_floor(myfloor, (int)dec_attempt_bucket(u));
                 n[u] = 0;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) n[u] += (uint32_t)__popcll(__ballot(a[s] >= f));
+                for (int s = 0; s < C; ++s) n[u] += (uint32_t)__popcll(__ballot(a[s] >= f));
             }
         }
         if (lane == 0) {
 #pragma unroll
-            for (int u = 0; u < kAttempts; ++u) wc[u * kSelWaves + tw] = n[u];
+            for (int u = 0; u < kAttempts; ++u) wc[u * 4 + tw] = n[u];
         }
     }
     __syncthreads();
     if (scanner) {
         // lane u < 8 looks at attempt u: total and the count of the team's waves before this one
-        const u32x4 w4 = *(const u32x4*)(wc + kSelWaves * (lane & 7u));
-        const uint32_t tot = w4[0] + w4[1] + w4[2] + w4[3];
+        const u32x4 w4 = *(const u32x4*)(wc + 4u * (lane & 7u));
+        const uint32_t tot = kSelWaves == 4u ? w4[0] + w4[1] + w4[2] + w4[3] : w4[0] + w4[1];
         const uint32_t before = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
-        const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= (uint32_t)kMaxCand);
+        const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= kCand);
         const bool fast = okm != 0ull;
         if (fast) {
             const uint32_t us = (uint32_t)__builtin_ctzll(okm);                     // first qualifying attempt
             const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)us);
             const uint32_t base = (uint32_t)__builtin_amdgcn_readlane((int)before, (int)us);
             const float f = dec_floor(myfloor, (int)dec_attempt_bucket_rt(us));
-            uint32_t cs[4], mine = 0;
+            uint32_t cs[C], mine = 0;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) { cs[s] = (mag(s) >= f) ? 1u : 0u; mine += cs[s]; }
+            for (int s = 0; s < C; ++s) { cs[s] = (mag(s) >= f) ? 1u : 0u; mine += cs[s]; }
             uint32_t idx = base + wave_scan(mine) - mine;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
+            for (int s = 0; s < C; ++s) {
                 if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
             }
             if (ttid == 0) { hdr[1] = total; hdr[2] = dec_attempt_bucket_rt(us); }
@@ -313,7 +332,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     bool any_big = false, any_general = false;
 #pragma unroll
     for (uint32_t j = 0; j < kTeams; ++j) {
-        const u32x2 h = *(const u32x2*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)(32 + 2 * kMaxCand) * 4);
+        const u32x2 h = *(const u32x2*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)T::kHdrWord * 4);
         any_general = any_general || h[0] == kTeamGeneral;
         any_big = any_big || (h[0] == kTeamFast && h[1] > (uint32_t)kWave);
     }
@@ -328,7 +347,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
         // trip through LDS beyond reading the candidate itself.  Team j ranks on its wave j: waves w and w + 4 of a
         // workgroup share a SIMD, so the ranking waves of the four teams sit on four different SIMDs (a single
         // wave issues an instruction every four cycles at best; four ranking waves on one SIMD took 2.2x as long).
-        if (tw == (team & (uint32_t)(kSelWaves - 1))) {
+        if (tw == (team & (kSelWaves - 1u))) {
             const bool valid = lane < total;
             const float xs = valid ? cx[lane] : 0.f;
             const uint32_t chl = valid ? key[lane] : 0u;
@@ -379,7 +398,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
         if (big) {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per team wave and step
             const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
 #pragma unroll 1
-            for (uint32_t tile = tw; tile < ntiles; tile += (uint32_t)kSelWaves) {
+            for (uint32_t tile = tw; tile < ntiles; tile += kSelWaves) {
                 const uint32_t jg = tile % njg, iq = tile / njg;
                 const uint32_t j = jg * 64u + lane;
                 const uint32_t mykey = j < total ? key[j] : 0u;
@@ -390,7 +409,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
                     const u32x4 k4 = kp[v];
                     r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
                 }
-                pc[iq * kMaxCand + j] = (uint8_t)r;
+                pc[iq * kCand + j] = (uint8_t)r;
             }
         }
         __syncthreads();
@@ -398,7 +417,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             const uint32_t niq = (total + 15u) >> 4;
             uint32_t pos = 0;
 #pragma unroll 4
-            for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kMaxCand + ttid];
+            for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kCand + ttid];
             if (pos < kc) {
                 const uint32_t ch = lo + (key[ttid] & 1023u);
                 const float xs = cx[ttid];
@@ -416,7 +435,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     if (any_general) {                                     // uniform for the workgroup; rare
 #pragma unroll 1
         for (uint32_t j = 0; j < kTeams; ++j) {
-            const uint32_t st = *(const uint32_t*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)(32 + 2 * kMaxCand) * 4);
+            const uint32_t st = *(const uint32_t*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)T::kHdrWord * 4);
             if (st != kTeamGeneral) continue;              // uniform
             const uint32_t tj = t0 + j, cj = cgid + tj * p.cg;
             const uint32_t kcj = p.k_chunk * dec_chunk_len(p, cj) / kChunk;
@@ -548,15 +567,16 @@ __device__ __forceinline__ void dec_role(const DecParams& p, uint32_t bid, unsig
     dec_stamp(p, bid, 0);
     // the teams ask for the activations of their first chunks before anything else: their latency is the
     // head of the critical path
-    constexpr uint32_t kTeams = (uint32_t)NW / kSelWaves;
+    using T = DecTeam<NW>;
+    constexpr uint32_t kTeams = T::kTeams, kTeamThreads = T::kThreads;
     const uint32_t nlocal = cgid < p.num_chunks ? (p.num_chunks - cgid + p.cg - 1u) / p.cg : 0u;   // chunks cgid, cgid + cg, ...
     const float myfloor = p.floors[tid & 31u];
-    uint32_t xpre[4] = {0u, 0u, 0u, 0u};
-    const uint32_t team0 = tid / (uint32_t)kTeamThreads;
+    uint32_t xpre[T::kLaneChannels] = {};
+    const uint32_t team0 = tid / kTeamThreads;
     const bool have_xpre = p.fused_select && p.monotone;                              // uniform
     if (have_xpre && team0 < nlocal) {
         const uint32_t c = cgid + team0 * p.cg;
-        dec_load_x4<DT>(p, c * kChunk, dec_chunk_len(p, c), 4u * (tid & (uint32_t)(kTeamThreads - 1)), xpre);
+        dec_load_x<DT, T::kLaneChannels>(p, c * kChunk, dec_chunk_len(p, c), (uint32_t)T::kLaneChannels * (tid & (kTeamThreads - 1u)), xpre);
     }
     for (uint32_t i = tid; i < p.slots_per_block; i += (uint32_t)NW * kWave) lrows[i] = -1;
     uint32_t nslots = 0;
