@@ -67,6 +67,22 @@ __device__ __forceinline__ float dec_floor(float myfloor, int i) {
     return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(myfloor), i));
 }
 
+// Bucket of |x| = ca when the floors do not increase: the number of floors strictly above ca, at most 31 (the callers'
+// candidates lie at or above some floor).  "Floor i is above ca" then holds for a prefix of the floors, so five
+// lane-indexed reads of the floor register (ds_bpermute: a cross-lane gather, no memory) find its length; a scan
+// over the floors with v_readlane is six times as many dependent steps for the single wave that ranks.
+// Needs every lane of the wave active.
+__device__ __forceinline__ uint32_t dec_bucket_of(float myfloor, float ca) {
+    uint32_t b = 0;
+#pragma unroll
+    for (uint32_t step = 16u; step >= 1u; step >>= 1) {
+        const float f = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute((int)((b + step - 1u) << 2),
+                                                                              (int)__float_as_uint(myfloor)));
+        b += (ca < f) ? step : 0u;
+    }
+    return b;
+}
+
 // ---- selection of one chunk ------------------------------------------------------------------
 // General path: every wave tests its 64 channels against all 32 buckets (one ballot per bucket),
 // per-(bucket, wave) counts are prefix-summed, and each member computes its position.  Exact for any
@@ -175,7 +191,7 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // All teams run through the same workgroup barriers; what a team does between them depends on its own
 // chunk only.  A chunk the fast path cannot take (non-monotone floors, more than kMaxCand candidates,
 // k_chunk > kMaxCand) is afterwards selected by the whole workgroup on the general path.
-constexpr int kAttempts = 8;
+constexpr int kAttempts = 9;
 // Team geometry by workgroup size.  A 16-wave workgroup has four teams of four waves (four channels per lane, up to
 // 256 candidates per chunk on the fast path); smaller workgroups have teams of two waves (eight channels per lane,
 // up to 128 candidates): an 8-wave workgroup then still selects four chunks at a time, a 4-wave one two.
@@ -187,8 +203,8 @@ template <int NW> struct DecTeam {
     static constexpr int kCand = NW >= 16 ? kMaxCand : kMaxCand / 2;   // fast-path candidate capacity: one per team thread
     // per-team LDS: candidate counts [kAttempts][4], keys [kCand], activations [kCand], header (state, candidate
     // count, bucket of the winning cut-off; padded), partial ranks [kCand / 16][kCand] bytes
-    static constexpr int kWords = 32 + 2 * kCand + 8;
-    static constexpr int kHdrWord = 32 + 2 * kCand;
+    static constexpr int kWords = 4 * kAttempts + 2 * kCand + 8;
+    static constexpr int kHdrWord = 4 * kAttempts + 2 * kCand;
     static constexpr size_t kBytes = (size_t)kWords * 4 + (size_t)(kCand / 16) * kCand;
 };
 __host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves) {
@@ -198,17 +214,14 @@ __host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves) {
 }
 enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u };
 
-// The cut-offs tried: every bucket just below the calibrated threshold (floor[15] = thresholds[k - 1]: with
-// activations like the calibration set about kc channels lie above it, and one bucket further down adds about
-// kc / 2 more, so the first window that holds kc channels rarely holds more than 64), coarser further down.
-__device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) {
-    return u == 0 ? 15u : u == 1 ? 16u : u == 2 ? 17u : u == 3 ? 18u : u == 4 ? 20u : u == 5 ? 23u : u == 6 ? 27u : 31u;
-}
-// the same for a wave-uniform run-time attempt number: one byte per attempt
-__device__ __forceinline__ uint32_t dec_attempt_bucket_rt(uint32_t u) {
-    const unsigned long long tab = 0x1F1B17141211100Full;   // bytes 15, 16, 17, 18, 20, 23, 27, 31
-    return (uint32_t)(tab >> (8u * u)) & 0xFFu;
-}
+// The cut-offs tried: buckets 15, 17, ..., 31.  floor[15] = thresholds[k - 1]: with activations like the calibration
+// set about kc channels lie above it and one bucket further down adds about kc / 2 more; activations weaker than the
+// calibration set (a decode step against thresholds taken from prefill) put the cut anywhere below.  Steps of two
+// buckets keep the first window that holds kc channels at or below 64 channels (the capacity of the single-wave
+// ranking) in the calibrated case and within kCand everywhere (steps of three at the low end sent a decoder's
+// output projection to the general path); a cut-off at every bucket cost every launch a microsecond of scanning.
+// A window of more than kCand channels, or none, leaves the chunk to the general path.
+__device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) { return 15u + 2u * u; }
 
 // The activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
 // costs a branch and a full wait each).
@@ -252,7 +265,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
 
     unsigned char* tbase = (unsigned char*)red + (size_t)team * kTeamBytes;
     uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][4] candidate counts (kSelWaves used)
-    uint32_t* key = wc + 32;                               // [kCand]
+    uint32_t* key = wc + 4 * kAttempts;                    // [kCand]
     float* cx = (float*)(key + kCand);                     // [kCand]
     uint32_t* hdr = wc + T::kHdrWord;                      // state, candidate count, bucket of the winning cut-off
     uint8_t* pc = tbase + (size_t)T::kWords * 4;           // [kCand / 16][kCand] partial ranks (each at most 16)
@@ -301,8 +314,8 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     }
     __syncthreads();
     if (scanner) {
-        // lane u < 8 looks at attempt u: total and the count of the team's waves before this one
-        const u32x4 w4 = *(const u32x4*)(wc + 4u * (lane & 7u));
+        // lane u < kAttempts looks at attempt u: total and the count of the team's waves before this one
+        const u32x4 w4 = *(const u32x4*)(wc + 4u * (lane < (uint32_t)kAttempts ? lane : 0u));
         const uint32_t tot = kSelWaves == 4u ? w4[0] + w4[1] + w4[2] + w4[3] : w4[0] + w4[1];
         const uint32_t before = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
         const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= kCand);
@@ -311,7 +324,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             const uint32_t us = (uint32_t)__builtin_ctzll(okm);                     // first qualifying attempt
             const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)us);
             const uint32_t base = (uint32_t)__builtin_amdgcn_readlane((int)before, (int)us);
-            const float f = dec_floor(myfloor, (int)dec_attempt_bucket_rt(us));
+            const float f = dec_floor(myfloor, (int)dec_attempt_bucket(us));
             uint32_t cs[C], mine = 0;
 #pragma unroll
             for (int s = 0; s < C; ++s) { cs[s] = (mag(s) >= f) ? 1u : 0u; mine += cs[s]; }
@@ -320,7 +333,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             for (int s = 0; s < C; ++s) {
                 if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
             }
-            if (ttid == 0) { hdr[1] = total; hdr[2] = dec_attempt_bucket_rt(us); }
+            if (ttid == 0) hdr[1] = total;
         }
         if (ttid == 0) hdr[0] = fast ? kTeamFast : kTeamGeneral;
     } else if (ttid == 0) {
@@ -352,12 +365,8 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             const float xs = valid ? cx[lane] : 0.f;
             const uint32_t chl = valid ? key[lane] : 0u;
             const float ca = __builtin_fabsf(xs);
-            // bucket = number of floors above the candidate; candidates lie at or above the winning cut-off
-            // floor[hd[2]], so later (smaller) floors cannot be above them
-            const uint32_t nfl = hd[2] + 1u;                   // uniform
-            uint32_t bkt = 0;
-#pragma unroll 1
-            for (uint32_t i = 0; i < nfl; ++i) bkt += (ca < dec_floor(myfloor, (int)i)) ? 1u : 0u;
+            // bucket = number of floors above the candidate (candidates lie at or above the winning cut-off)
+            const uint32_t bkt = dec_bucket_of(myfloor, ca);
             unsigned long long eq = total >= 64u ? ~0ull : ((1ull << total) - 1ull);    // lanes whose bucket equals mine
             unsigned long long lt = 0ull;                                               // lanes whose bucket is lower
 #pragma unroll
@@ -384,11 +393,8 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
         const bool big = fast && total > (uint32_t)kWave;  // uniform per team
         // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
         if (big && __builtin_amdgcn_readfirstlane(ttid & ~63u) < total) {
+            const uint32_t bkt = dec_bucket_of(myfloor, ttid < total ? __builtin_fabsf(cx[ttid]) : 0.f);
             if (ttid < total) {
-                const float ca = __builtin_fabsf(cx[ttid]);
-                uint32_t bkt = 0;
-#pragma unroll
-                for (int i = 0; i < kBuckets; ++i) bkt += (ca < dec_floor(myfloor, i)) ? 1u : 0u;
                 key[ttid] |= bkt << 10;
             } else if (ttid < ((total + 15u) & ~15u)) {
                 key[ttid] = 0xFFFFFFFFu;                   // padding of the last 16-key tile: never smaller
