@@ -176,51 +176,60 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 }
 
 // Fast path (floors finite and non-increasing, checked on the host).  Then bucket(|x|) is the number of
-// floors above |x|, buckets 0..T tile [floor_T, +inf), and as soon as at least kc channels lie in that
-// range they are the only possible picks.  Eight cut-offs T are tried at once (a compare and a ballot
-// each); the first whose range holds at least kc and at most kMaxCand channels wins.  Those candidates
-// (usually a few dozen of 1024) are compacted in channel order, get the key (bucket << 10 | channel),
-// and the canonical position of a candidate is the number of smaller keys, counted all-pairs.  No
-// sequential walk over buckets.
+// floors above |x|, buckets 0..T tile [floor_T, +inf), and the selection is: every channel of the buckets before
+// the cut bucket b* (the first bucket at which the running count reaches kc), then the first channels of b* in
+// channel order.  kAttempts cut-offs T are tried at once (a compare and a ballot each); the first whose range holds
+// at least kc channels is the winning window.
+//   * At most 64 channels in the window (the usual case): they are compacted in channel order and one wave ranks
+//     them by (bucket, channel) with ballots.
+//   * More (activations weaker than the calibration set put the cut where buckets are crowded): the window spans two
+//     buckets beyond the previous cut-off; one more count at the floor between them tells which of the two is b*.
+//     The channels above b* -- fewer than kc, so at most 63 -- are compacted and ranked as before; the members of
+//     b* need no ranking at all: their positions follow the ranked ones in channel order, so each writes its own
+//     output slot from a prefix count, however many there are.
+// No sequential walk over buckets, and no limit on the size of a bucket.
 //
 // A wave issues one instruction every four cycles whatever its kind, so a chunk is scanned by a TEAM of
-// four waves (one per SIMD, four channels per lane).  The teams of a workgroup (four in a 1024-thread
-// workgroup) take different chunks of the workgroup's chunk list at the same time: a workgroup that owns
-// up to four chunks selects them in the time of one, which is what lets the launch plan give a workgroup
-// several chunks (few chunk groups = few atomic adds, i.e. roundings, per output) at no cost in latency.
-// All teams run through the same workgroup barriers; what a team does between them depends on its own
-// chunk only.  A chunk the fast path cannot take (non-monotone floors, more than kMaxCand candidates,
-// k_chunk > kMaxCand) is afterwards selected by the whole workgroup on the general path.
+// waves on different SIMDs.  The teams of a workgroup (four in a 1024-thread workgroup) take different chunks of
+// the workgroup's chunk list at the same time: a workgroup that owns up to four chunks selects them in the time of
+// one, which is what lets the launch plan give a workgroup several chunks (few chunk groups = few atomic adds,
+// i.e. roundings, per output) at no cost in latency.  All teams run through the same workgroup barriers; what a
+// team does between them depends on its own chunk only.  A chunk the fast path cannot take (non-monotone floors,
+// k_chunk > 64, NaN or infinite activations that leave fewer than kc countable channels, more than 64 channels in
+// the buckets down to the calibrated threshold) is afterwards selected by the whole workgroup on the general path.
 constexpr int kAttempts = 9;
-// Team geometry by workgroup size.  A 16-wave workgroup has four teams of four waves (four channels per lane, up to
-// 256 candidates per chunk on the fast path); smaller workgroups have teams of two waves (eight channels per lane,
-// up to 128 candidates): an 8-wave workgroup then still selects four chunks at a time, a 4-wave one two.
+constexpr uint32_t kRankMax = 64;          // candidates one wave ranks
+// Team geometry by workgroup size.  A 16-wave workgroup has four teams of four waves (four channels per lane);
+// smaller workgroups have teams of two waves (eight channels per lane): an 8-wave workgroup then still selects
+// four chunks at a time, a 4-wave one two.
 template <int NW> struct DecTeam {
     static constexpr int kWaves = NW >= 16 ? 4 : 2;                 // waves of a team
     static constexpr int kThreads = kWaves * kWave;
     static constexpr int kTeams = NW / kWaves;
-    static constexpr int kLaneChannels = kChunk / kThreads;        // channels a scanning lane owns: 4 or 8
-    static constexpr int kCand = NW >= 16 ? kMaxCand : kMaxCand / 2;   // fast-path candidate capacity: one per team thread
-    // per-team LDS: candidate counts [kAttempts][4], keys [kCand], activations [kCand], header (state, candidate
-    // count, bucket of the winning cut-off; padded), partial ranks [kCand / 16][kCand] bytes
-    static constexpr int kWords = 4 * kAttempts + 2 * kCand + 8;
-    static constexpr int kHdrWord = 4 * kAttempts + 2 * kCand;
-    static constexpr size_t kBytes = (size_t)kWords * 4 + (size_t)(kCand / 16) * kCand;
+    static constexpr int kLaneChannels = kChunk / kThreads;         // 4 or 8
+    // Crowded windows are split only in the 16-wave workgroups.  The smaller ones share their kernel, and its
+    // register allocation, with a GEMV role that runs eight waves per SIMD; they are chosen while DEC is the
+    // shorter role, and leave the rare crowded window to the general path.
+    static constexpr bool kSplit = NW >= 16;
+    // words of a team's area: [kAttempts][4] window counts, [4] counts at the floor inside the window,
+    // [64] candidate channels, [64] candidate activations, [4] header (state, candidates, -, -)
+    static constexpr int kSplitWord = 4 * kAttempts;
+    static constexpr int kKeyWord = kSplitWord + 4;
+    static constexpr int kHdrWord = kKeyWord + 2 * (int)kRankMax;
+    static constexpr size_t kBytes = (size_t)(kHdrWord + 4) * 4;
+    static_assert(kBytes % 16 == 0 && (kKeyWord * 4) % 16 == 0 && (kHdrWord * 4) % 16 == 0, "team area alignment");
 };
 __host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves) {
     return nwaves >= 16 ? (size_t)DecTeam<16>::kTeams * DecTeam<16>::kBytes
                         : (nwaves >= 8 ? (size_t)DecTeam<8>::kTeams * DecTeam<8>::kBytes
                                        : (size_t)DecTeam<4>::kTeams * DecTeam<4>::kBytes);
 }
-enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u };
+enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u, kTeamSplit = 3u };
 
 // The cut-offs tried: buckets 15, 17, ..., 31.  floor[15] = thresholds[k - 1]: with activations like the calibration
-// set about kc channels lie above it and one bucket further down adds about kc / 2 more; activations weaker than the
-// calibration set (a decode step against thresholds taken from prefill) put the cut anywhere below.  Steps of two
-// buckets keep the first window that holds kc channels at or below 64 channels (the capacity of the single-wave
-// ranking) in the calibrated case and within kCand everywhere (steps of three at the low end sent a decoder's
-// output projection to the general path); a cut-off at every bucket cost every launch a microsecond of scanning.
-// A window of more than kCand channels, or none, leaves the chunk to the general path.
+// set about kc channels lie above it and one bucket further down adds about kc / 2 more, so steps of two buckets keep
+// the winning window at or below 64 channels there; a cut-off at every bucket cost every launch a microsecond of
+// scanning.  floor[31] = 0: the last window always holds every finite channel.
 __device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) { return 15u + 2u * u; }
 
 // The activations a scanning lane owns: unconditional loads from clamped indices (a predicated load
@@ -237,6 +246,36 @@ __device__ __forceinline__ uint32_t dec_chunk_len(const DecParams& p, uint32_t c
     return (p.K - lo) < (uint32_t)kChunk ? (p.K - lo) : (uint32_t)kChunk;
 }
 
+// What a team's window counts say (the same in every lane of every wave of the team).
+struct DecWindow {
+    uint32_t state;        // kTeamFast, kTeamSplit or kTeamGeneral
+    uint32_t us;           // winning attempt
+    uint32_t total;        // channels in the winning window (all buckets down to its cut-off)
+    uint32_t before;       // ... of them in the team's waves before this one
+    uint32_t prev_total;   // channels above the previous cut-off (0 for the first attempt): fewer than kc
+    uint32_t prev_before;
+};
+template <int NW>
+__device__ __forceinline__ DecWindow dec_read_window(const uint32_t* wc, uint32_t lane, uint32_t tw, uint32_t kc) {
+    constexpr uint32_t kSelWaves = DecTeam<NW>::kWaves;
+    // lane u < kAttempts looks at attempt u: total and the count of the team's waves before this one
+    const u32x4 w4 = *(const u32x4*)(wc + 4u * (lane < (uint32_t)kAttempts ? lane : 0u));
+    const uint32_t tot = kSelWaves == 4u ? w4[0] + w4[1] + w4[2] + w4[3] : w4[0] + w4[1];
+    const uint32_t bef = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
+    const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc);
+    DecWindow w = {kTeamGeneral, 0u, 0u, 0u, 0u, 0u};
+    if (okm == 0ull || kc > kRankMax) return w;
+    w.us = (uint32_t)__builtin_ctzll(okm);                                          // first qualifying attempt
+    w.total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)w.us);
+    w.before = (uint32_t)__builtin_amdgcn_readlane((int)bef, (int)w.us);
+    if (w.us > 0u) {
+        w.prev_total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)w.us - 1);
+        w.prev_before = (uint32_t)__builtin_amdgcn_readlane((int)bef, (int)w.us - 1);
+    }
+    w.state = w.total <= kRankMax ? kTeamFast : ((DecTeam<NW>::kSplit && w.us > 0u) ? kTeamSplit : kTeamGeneral);
+    return w;
+}
+
 // One round of selection: team j of the workgroup takes the workgroup's local chunk t0 + j (global chunk
 // cgid + (t0 + j) * cg) if there is one.  `xpre` holds the raw activations of the team's chunk when
 // have_xpre (requested when the workgroup started).  Called by all threads of the workgroup.
@@ -248,7 +287,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
                                                  const float myfloor) {
     using E = Elem<DT>;
     using T = DecTeam<NW>;
-    constexpr uint32_t kTeams = T::kTeams, kSelWaves = T::kWaves, kTeamThreads = T::kThreads, kCand = T::kCand;
+    constexpr uint32_t kTeams = T::kTeams, kSelWaves = T::kWaves, kTeamThreads = T::kThreads;
     constexpr int C = T::kLaneChannels;
     constexpr size_t kTeamBytes = T::kBytes;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -264,22 +303,53 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     const bool active = has_chunk && kc > 0u;
 
     unsigned char* tbase = (unsigned char*)red + (size_t)team * kTeamBytes;
-    uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][4] candidate counts (kSelWaves used)
-    uint32_t* key = wc + 4 * kAttempts;                    // [kCand]
-    float* cx = (float*)(key + kCand);                     // [kCand]
-    uint32_t* hdr = wc + T::kHdrWord;                      // state, candidate count, bucket of the winning cut-off
-    uint8_t* pc = tbase + (size_t)T::kWords * 4;           // [kCand / 16][kCand] partial ranks (each at most 16)
+    uint32_t* wc = (uint32_t*)tbase;                       // [kAttempts][4] window counts per team wave
+    uint32_t* split = wc + T::kSplitWord;                  // [4] counts at the floor inside the winning window
+    uint32_t* key = wc + T::kKeyWord;                      // [kRankMax] candidate channels (chunk-relative)
+    float* cx = (float*)(key + kRankMax);                  // [kRankMax] their activations
+    uint32_t* hdr = wc + T::kHdrWord;                      // state, candidates to rank
     const bool scanner = active && p.monotone;             // uniform per wave
 
     // ---- the team scans its chunk: lane l of team wave w owns channels C (64 w + l) .. + C - 1
     // |x| of the lane's channel s as the selection sees it: NaN, inf and channels past the end are members of no
-    // bucket.  Recomputed after the barrier instead of kept: registers held across it are charged to every kernel
-    // that contains this role.
+    // bucket.  Recomputed after the barriers instead of kept: registers held across them are charged to every
+    // kernel that contains this role.
     float xv[C];
     const uint32_t ch0 = (uint32_t)C * ttid;
     auto mag = [&](int s) {
         const float v = __builtin_fabsf(xv[s]);
         return (ch0 + (uint32_t)s < len && v < __builtin_inff()) ? v : -__builtin_inff();
+    };
+    // selected channel at canonical position pos of the team's chunk
+    auto emit = [&](uint32_t pos, uint32_t chl, float xs) {
+        const uint32_t ch = lo + chl;
+        const uint32_t slot = t_local * p.k_chunk + pos;
+        lrows[slot] = (int32_t)ch;
+        lacts[slot] = xs;
+        if (write_global) {
+            p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
+            E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
+        }
+    };
+    // The candidates in key / cx (n of them, in channel order, n <= 64) ranked by (bucket, channel) by the calling
+    // wave with ballots only: a candidate's position is the number of candidates in lower buckets plus the number of
+    // earlier lanes in its own bucket.  The first min(n, kc) positions are emitted.
+    auto rank_candidates = [&](uint32_t n) {
+        const bool valid = lane < n;
+        const float xs = valid ? cx[lane] : 0.f;
+        const uint32_t chl = valid ? key[lane] : 0u;
+        const uint32_t bkt = dec_bucket_of(myfloor, __builtin_fabsf(xs));
+        unsigned long long eq = n >= 64u ? ~0ull : ((1ull << n) - 1ull);    // lanes whose bucket equals mine
+        unsigned long long lt = 0ull;                                       // lanes whose bucket is lower
+#pragma unroll
+        for (int k = 4; k >= 0; --k) {
+            const bool mybit = ((bkt >> k) & 1u) != 0u;
+            const unsigned long long bk = __ballot(valid && mybit);
+            lt |= mybit ? (eq & ~bk) : 0ull;
+            eq &= mybit ? bk : ~bk;
+        }
+        const uint32_t pos = (uint32_t)__popcll(lt) + ballot_rank(eq);
+        if (valid && pos < kc) emit(pos, chl, xs);
     };
     if (scanner) {
         uint32_t xr[C];
@@ -314,128 +384,77 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     }
     __syncthreads();
     if (scanner) {
-        // lane u < kAttempts looks at attempt u: total and the count of the team's waves before this one
-        const u32x4 w4 = *(const u32x4*)(wc + 4u * (lane < (uint32_t)kAttempts ? lane : 0u));
-        const uint32_t tot = kSelWaves == 4u ? w4[0] + w4[1] + w4[2] + w4[3] : w4[0] + w4[1];
-        const uint32_t before = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
-        const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc && tot <= kCand);
-        const bool fast = okm != 0ull;
-        if (fast) {
-            const uint32_t us = (uint32_t)__builtin_ctzll(okm);                     // first qualifying attempt
-            const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)us);
-            const uint32_t base = (uint32_t)__builtin_amdgcn_readlane((int)before, (int)us);
-            const float f = dec_floor(myfloor, (int)dec_attempt_bucket(us));
+        const DecWindow w = dec_read_window<NW>(wc, lane, tw, kc);
+        if (w.state == kTeamFast) {                        // compaction of the window in channel order
+            const float f = dec_floor(myfloor, (int)dec_attempt_bucket(w.us));
             uint32_t cs[C], mine = 0;
 #pragma unroll
             for (int s = 0; s < C; ++s) { cs[s] = (mag(s) >= f) ? 1u : 0u; mine += cs[s]; }
-            uint32_t idx = base + wave_scan(mine) - mine;
+            uint32_t idx = w.before + wave_scan(mine) - mine;
 #pragma unroll
             for (int s = 0; s < C; ++s) {
                 if (cs[s]) { key[idx] = ch0 + s; cx[idx] = xv[s]; ++idx; }
             }
-            if (ttid == 0) hdr[1] = total;
+            if (ttid == 0) hdr[1] = w.total;
+        } else if (w.state == kTeamSplit) {                // channels at or above the floor inside the window
+            const float f = dec_floor(myfloor, (int)dec_attempt_bucket(w.us) - 1);
+            uint32_t nu = 0;
+#pragma unroll
+            for (int s = 0; s < C; ++s) nu += (uint32_t)__popcll(__ballot(mag(s) >= f));
+            if (lane == 0) split[tw] = nu;
         }
-        if (ttid == 0) hdr[0] = fast ? kTeamFast : kTeamGeneral;
+        if (ttid == 0) hdr[0] = w.state;
     } else if (ttid == 0) {
         hdr[0] = active ? kTeamGeneral : kTeamIdle;
         hdr[1] = 0u;
     }
     __syncthreads();
     // what the teams found (the same view in every thread: the branches below that hold barriers are uniform)
-    bool any_big = false, any_general = false;
+    bool any_split = false, any_general = false;
 #pragma unroll
     for (uint32_t j = 0; j < kTeams; ++j) {
-        const u32x2 h = *(const u32x2*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)T::kHdrWord * 4);
-        any_general = any_general || h[0] == kTeamGeneral;
-        any_big = any_big || (h[0] == kTeamFast && h[1] > (uint32_t)kWave);
+        const uint32_t st = *(const uint32_t*)((const unsigned char*)red + (size_t)j * kTeamBytes + (size_t)T::kHdrWord * 4);
+        any_general = any_general || st == kTeamGeneral;
+        any_split = any_split || st == kTeamSplit;
     }
-    const u32x4 hd = *(const u32x4*)hdr;                    // state, candidates, bucket of the winning cut-off
-    const bool fast = hd[0] == kTeamFast;
-    const uint32_t total = hd[1];
+    const u32x2 hd = *(const u32x2*)hdr;                    // state, candidates
     dec_stamp(p, blockIdx.x, 6);
-    if (fast && total <= (uint32_t)kWave) {
-        // The usual case: at most 64 candidates, in channel order.  One wave holds a candidate per lane and ranks
-        // them by (bucket, channel) with ballots only: a candidate's position is the number of candidates in lower
-        // buckets plus the number of earlier lanes in its own bucket.  Nothing here needs a workgroup barrier or a
-        // trip through LDS beyond reading the candidate itself.  Team j ranks on its wave j: waves w and w + 4 of a
-        // workgroup share a SIMD, so the ranking waves of the four teams sit on four different SIMDs (a single
-        // wave issues an instruction every four cycles at best; four ranking waves on one SIMD took 2.2x as long).
-        if (tw == (team & (kSelWaves - 1u))) {
-            const bool valid = lane < total;
-            const float xs = valid ? cx[lane] : 0.f;
-            const uint32_t chl = valid ? key[lane] : 0u;
-            const float ca = __builtin_fabsf(xs);
-            // bucket = number of floors above the candidate (candidates lie at or above the winning cut-off)
-            const uint32_t bkt = dec_bucket_of(myfloor, ca);
-            unsigned long long eq = total >= 64u ? ~0ull : ((1ull << total) - 1ull);    // lanes whose bucket equals mine
-            unsigned long long lt = 0ull;                                               // lanes whose bucket is lower
+    // Team j ranks on its wave j: waves w and w + 4 of a workgroup share a SIMD, so the ranking waves of the four
+    // teams sit on four different SIMDs (four ranking waves on one SIMD took 2.2x as long).
+    const bool ranker = tw == (team & (kSelWaves - 1u));
+    if (hd[0] == kTeamFast && ranker) rank_candidates(hd[1]);
+    if (T::kSplit && any_split) {                          // uniform for the workgroup
+        if (hd[0] == kTeamSplit) {                         // uniform per team
+            const DecWindow w = dec_read_window<NW>(wc, lane, tw, kc);
+            const u32x4 s4 = *(const u32x4*)split;
+            const uint32_t stot = kSelWaves == 4u ? s4[0] + s4[1] + s4[2] + s4[3] : s4[0] + s4[1];
+            const uint32_t sbef = (tw > 0 ? s4[0] : 0u) + (tw > 1 ? s4[1] : 0u) + (tw > 2 ? s4[2] : 0u);
+            // the cut bucket is the upper one of the window's two if the count reaches kc there, else the lower one
+            const bool upper = stot >= kc;
+            const uint32_t bb = dec_attempt_bucket(w.us) - (upper ? 1u : 0u);                       // cut bucket
+            const float fb = dec_floor(myfloor, (int)bb), fs = dec_floor(myfloor, (int)bb - 1);
+            const uint32_t n_sure = upper ? w.prev_total : stot;                                   // < kc
+            const uint32_t sure_before = upper ? w.prev_before : sbef;
+            const uint32_t band_before = (upper ? sbef : w.before) - sure_before;
+            uint32_t cs[C], cb[C], ms = 0, mb = 0;
 #pragma unroll
-            for (int k = 4; k >= 0; --k) {
-                const bool mybit = ((bkt >> k) & 1u) != 0u;
-                const unsigned long long bk = __ballot(valid && mybit);
-                lt |= mybit ? (eq & ~bk) : 0ull;
-                eq &= mybit ? bk : ~bk;
+            for (int s = 0; s < C; ++s) {
+                const float a = mag(s);
+                cs[s] = (a >= fs) ? 1u : 0u;
+                cb[s] = (a >= fb && !(a >= fs)) ? 1u : 0u;
+                ms += cs[s]; mb += cb[s];
             }
-            const uint32_t pos = (uint32_t)__popcll(lt) + ballot_rank(eq);
-            if (valid && pos < kc) {
-                const uint32_t ch = lo + chl;
-                const uint32_t slot = t_local * p.k_chunk + pos;
-                lrows[slot] = (int32_t)ch;
-                lacts[slot] = xs;
-                if (write_global) {
-                    p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
-                    E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
-                }
+            uint32_t is = sure_before + wave_scan(ms) - ms;
+            uint32_t ib = n_sure + band_before + wave_scan(mb) - mb;
+#pragma unroll
+            for (int s = 0; s < C; ++s) {
+                if (cs[s]) { key[is] = ch0 + s; cx[is] = xv[s]; ++is; }
+                if (cb[s]) { if (ib < kc) emit(ib, ch0 + s, xv[s]); ++ib; }
             }
-        }
-    }
-    if (any_big) {                                         // uniform for the workgroup
-        const bool big = fast && total > (uint32_t)kWave;  // uniform per team
-        // bucket of every candidate = number of floors strictly above it (none below the cut-off can be)
-        if (big && __builtin_amdgcn_readfirstlane(ttid & ~63u) < total) {
-            const uint32_t bkt = dec_bucket_of(myfloor, ttid < total ? __builtin_fabsf(cx[ttid]) : 0.f);
-            if (ttid < total) {
-                key[ttid] |= bkt << 10;
-            } else if (ttid < ((total + 15u) & ~15u)) {
-                key[ttid] = 0xFFFFFFFFu;                   // padding of the last 16-key tile: never smaller
-            }
+            if (ttid == 0) hdr[1] = n_sure;
         }
         __syncthreads();
-        if (big) {   // partial rank of candidate j among keys [16 iq, 16 iq + 16): one tile per team wave and step
-            const uint32_t njg = (total + 63u) >> 6, niq = (total + 15u) >> 4, ntiles = njg * niq;
-#pragma unroll 1
-            for (uint32_t tile = tw; tile < ntiles; tile += kSelWaves) {
-                const uint32_t jg = tile % njg, iq = tile / njg;
-                const uint32_t j = jg * 64u + lane;
-                const uint32_t mykey = j < total ? key[j] : 0u;
-                const u32x4* kp = (const u32x4*)(key + iq * 16u);
-                uint32_t r = 0;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const u32x4 k4 = kp[v];
-                    r += (k4[0] < mykey) + (k4[1] < mykey) + (k4[2] < mykey) + (k4[3] < mykey);
-                }
-                pc[iq * kCand + j] = (uint8_t)r;
-            }
-        }
-        __syncthreads();
-        if (big && __builtin_amdgcn_readfirstlane(ttid & ~63u) < total && ttid < total) {
-            const uint32_t niq = (total + 15u) >> 4;
-            uint32_t pos = 0;
-#pragma unroll 4
-            for (uint32_t iq = 0; iq < niq; ++iq) pos += pc[iq * kCand + ttid];
-            if (pos < kc) {
-                const uint32_t ch = lo + (key[ttid] & 1023u);
-                const float xs = cx[ttid];
-                const uint32_t slot = t_local * p.k_chunk + pos;
-                lrows[slot] = (int32_t)ch;
-                lacts[slot] = xs;
-                if (write_global) {
-                    p.sel_rows[(size_t)c * p.k_chunk + pos] = (int32_t)ch;
-                    E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
-                }
-            }
-        }
+        if (hd[0] == kTeamSplit && ranker) rank_candidates(hdr[1]);
     }
     dec_stamp(p, blockIdx.x, 7);
     if (any_general) {                                     // uniform for the workgroup; rare
