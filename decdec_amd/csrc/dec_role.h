@@ -48,8 +48,7 @@ __device__ __forceinline__ void dec_stamp(const DecParams& p, uint32_t bid, int 
 
 constexpr int kDecThreads = 1024;                            // largest DEC workgroup
 constexpr int kDecWaves = kDecThreads / kWave;
-constexpr int kMinDecWaves = 4;                              // smallest: the four scanning waves
-constexpr int kMaxCand = 256;                                // fast-path candidate list capacity
+constexpr int kMinDecWaves = 4;                              // smallest workgroup: two teams of two waves
 constexpr int kMergeTasks = kDecWaves * 256 / kDecThreads;   // output pairs per thread and segment batch
 
 __host__ __device__ inline size_t dec_team_lds_bytes(uint32_t nwaves);
@@ -180,11 +179,11 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // the cut bucket b* (the first bucket at which the running count reaches kc), then the first channels of b* in
 // channel order.  kAttempts cut-offs T are tried at once (a compare and a ballot each); the first whose range holds
 // at least kc channels is the winning window.
-//   * At most 64 channels in the window (the usual case): they are compacted in channel order and one wave ranks
-//     them by (bucket, channel) with ballots.
+//   * At most 128 channels in the window (64 in the usual case): they are compacted in channel order and one wave
+//     (two beyond 64) ranks them by (bucket, channel) with ballots.
 //   * More (activations weaker than the calibration set put the cut where buckets are crowded): the window spans two
 //     buckets beyond the previous cut-off; one more count at the floor between them tells which of the two is b*.
-//     The channels above b* -- fewer than kc, so at most 63 -- are compacted and ranked as before; the members of
+//     The channels above b* -- fewer than kc, so at most 127 -- are compacted and ranked as before; the members of
 //     b* need no ranking at all: their positions follow the ranked ones in channel order, so each writes its own
 //     output slot from a prefix count, however many there are.
 // No sequential walk over buckets, and no limit on the size of a bucket.
@@ -195,10 +194,10 @@ __device__ __forceinline__ uint32_t wave_scan(uint32_t v) {
 // one, which is what lets the launch plan give a workgroup several chunks (few chunk groups = few atomic adds,
 // i.e. roundings, per output) at no cost in latency.  All teams run through the same workgroup barriers; what a
 // team does between them depends on its own chunk only.  A chunk the fast path cannot take (non-monotone floors,
-// k_chunk > 64, NaN or infinite activations that leave fewer than kc countable channels, more than 64 channels in
+// k_chunk > 128, NaN or infinite activations that leave fewer than kc countable channels, more than 128 channels in
 // the buckets down to the calibrated threshold) is afterwards selected by the whole workgroup on the general path.
 constexpr int kAttempts = 9;
-constexpr uint32_t kRankMax = 64;          // candidates one wave ranks
+constexpr uint32_t kRankMax = 128;         // candidates a team of a 16-wave workgroup ranks (64 per ranking wave)
 // Team geometry by workgroup size.  A 16-wave workgroup has four teams of four waves (four channels per lane);
 // smaller workgroups have teams of two waves (eight channels per lane): an 8-wave workgroup then still selects
 // four chunks at a time, a 4-wave one two.
@@ -207,12 +206,14 @@ template <int NW> struct DecTeam {
     static constexpr int kThreads = kWaves * kWave;
     static constexpr int kTeams = NW / kWaves;
     static constexpr int kLaneChannels = kChunk / kThreads;         // 4 or 8
-    // Crowded windows are split only in the 16-wave workgroups.  The smaller ones share their kernel, and its
-    // register allocation, with a GEMV role that runs eight waves per SIMD; they are chosen while DEC is the
-    // shorter role, and leave the rare crowded window to the general path.
+    // Windows of more than 64 channels are ranked by two waves, and crowded ones split, only in the 16-wave
+    // workgroups.  The smaller ones share their kernel, and its register allocation, with a GEMV role that runs
+    // eight waves per SIMD (every addition to this role made that role slower); they are chosen while DEC is the
+    // shorter role, and leave the rare window of more than 64 channels to the general path.
     static constexpr bool kSplit = NW >= 16;
+    static constexpr uint32_t kRank = kSplit ? kRankMax : 64u;      // candidates a team ranks (64 per ranking wave)
     // words of a team's area: [kAttempts][4] window counts, [4] counts at the floor inside the window,
-    // [64] candidate channels, [64] candidate activations, [4] header (state, candidates, -, -)
+    // [kRankMax] candidate channels, [kRankMax] candidate activations, [4] header (state, candidates, -, -)
     static constexpr int kSplitWord = 4 * kAttempts;
     static constexpr int kKeyWord = kSplitWord + 4;
     static constexpr int kHdrWord = kKeyWord + 2 * (int)kRankMax;
@@ -228,7 +229,7 @@ enum : uint32_t { kTeamGeneral = 0u, kTeamFast = 1u, kTeamIdle = 2u, kTeamSplit 
 
 // The cut-offs tried: buckets 15, 17, ..., 31.  floor[15] = thresholds[k - 1]: with activations like the calibration
 // set about kc channels lie above it and one bucket further down adds about kc / 2 more, so steps of two buckets keep
-// the winning window at or below 64 channels there; a cut-off at every bucket cost every launch a microsecond of
+// the winning window at or below 64 channels (one ranking wave) there; a cut-off at every bucket cost every launch a microsecond of
 // scanning.  floor[31] = 0: the last window always holds every finite channel.
 __device__ __forceinline__ constexpr uint32_t dec_attempt_bucket(uint32_t u) { return 15u + 2u * u; }
 
@@ -264,7 +265,7 @@ __device__ __forceinline__ DecWindow dec_read_window(const uint32_t* wc, uint32_
     const uint32_t bef = (tw > 0 ? w4[0] : 0u) + (tw > 1 ? w4[1] : 0u) + (tw > 2 ? w4[2] : 0u);
     const unsigned long long okm = __ballot(lane < (uint32_t)kAttempts && tot >= kc);
     DecWindow w = {kTeamGeneral, 0u, 0u, 0u, 0u, 0u};
-    if (okm == 0ull || kc > kRankMax) return w;
+    if (okm == 0ull || kc > DecTeam<NW>::kRank) return w;
     w.us = (uint32_t)__builtin_ctzll(okm);                                          // first qualifying attempt
     w.total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)w.us);
     w.before = (uint32_t)__builtin_amdgcn_readlane((int)bef, (int)w.us);
@@ -272,7 +273,7 @@ __device__ __forceinline__ DecWindow dec_read_window(const uint32_t* wc, uint32_
         w.prev_total = (uint32_t)__builtin_amdgcn_readlane((int)tot, (int)w.us - 1);
         w.prev_before = (uint32_t)__builtin_amdgcn_readlane((int)bef, (int)w.us - 1);
     }
-    w.state = w.total <= kRankMax ? kTeamFast : ((DecTeam<NW>::kSplit && w.us > 0u) ? kTeamSplit : kTeamGeneral);
+    w.state = w.total <= DecTeam<NW>::kRank ? kTeamFast : ((DecTeam<NW>::kSplit && w.us > 0u) ? kTeamSplit : kTeamGeneral);
     return w;
 }
 
@@ -331,25 +332,54 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             E::store(p.sel_acts, (size_t)c * p.k_chunk + pos, xs);
         }
     };
-    // The candidates in key / cx (n of them, in channel order, n <= 64) ranked by (bucket, channel) by the calling
-    // wave with ballots only: a candidate's position is the number of candidates in lower buckets plus the number of
-    // earlier lanes in its own bucket.  The first min(n, kc) positions are emitted.
-    auto rank_candidates = [&](uint32_t n) {
-        const bool valid = lane < n;
-        const float xs = valid ? cx[lane] : 0.f;
-        const uint32_t chl = valid ? key[lane] : 0u;
-        const uint32_t bkt = dec_bucket_of(myfloor, __builtin_fabsf(xs));
-        unsigned long long eq = n >= 64u ? ~0ull : ((1ull << n) - 1ull);    // lanes whose bucket equals mine
-        unsigned long long lt = 0ull;                                       // lanes whose bucket is lower
+    // The candidates in key / cx (n of them, in channel order, n <= 128) ranked by (bucket, channel) with ballots only:
+    // a candidate's position is the number of candidates in lower buckets plus the number of earlier candidates in its
+    // own bucket.  A wave places the 64 candidates of half `half` (lane l holds candidate 64 half + l) and looks at
+    // both halves when there are more than 64; the first min(n, kc) positions are emitted.  Called by whole waves.
+    auto rank_candidates = [&](uint32_t n, uint32_t half) {
+        const uint32_t nh = (T::kRank > 64u && n > 64u) ? 2u : 1u;      // halves in use (uniform)
+        bool valid[2] = {false, false};
+        float xs[2] = {0.f, 0.f};
+        uint32_t chl[2] = {0u, 0u}, bkt[2] = {0u, 0u};
 #pragma unroll
-        for (int k = 4; k >= 0; --k) {
-            const bool mybit = ((bkt >> k) & 1u) != 0u;
-            const unsigned long long bk = __ballot(valid && mybit);
-            lt |= mybit ? (eq & ~bk) : 0ull;
-            eq &= mybit ? bk : ~bk;
+        for (uint32_t h = 0; h < 2u; ++h) {
+            if (h < nh) {
+                const uint32_t i = 64u * h + lane;
+                valid[h] = i < n;
+                xs[h] = valid[h] ? cx[i] : 0.f;
+                chl[h] = valid[h] ? key[i] : 0u;
+                bkt[h] = dec_bucket_of(myfloor, __builtin_fabsf(xs[h]));
+            }
         }
-        const uint32_t pos = (uint32_t)__popcll(lt) + ballot_rank(eq);
-        if (valid && pos < kc) emit(pos, chl, xs);
+        const uint32_t mybkt = half ? bkt[1] : bkt[0];
+        uint32_t pos = 0;
+#pragma unroll
+        for (uint32_t h = 0; h < 2u; ++h) {
+            if (h < nh) {
+                unsigned long long eq = __ballot(valid[h]);             // candidates of half h in my bucket
+                unsigned long long lt = 0ull;                           // ... in a lower bucket
+#pragma unroll
+                for (int k = 4; k >= 0; --k) {
+                    const bool mybit = ((mybkt >> k) & 1u) != 0u;
+                    const unsigned long long bk = __ballot(valid[h] && ((bkt[h] >> k) & 1u) != 0u);
+                    lt |= mybit ? (eq & ~bk) : 0ull;
+                    eq &= mybit ? bk : ~bk;
+                }
+                pos += (uint32_t)__popcll(lt);
+                // same bucket: all of an earlier half, the earlier lanes of my own half, none of a later half
+                pos += h < half ? (uint32_t)__popcll(eq) : (h == half ? ballot_rank(eq) : 0u);
+            }
+        }
+        const bool myvalid = half ? valid[1] : valid[0];
+        if (myvalid && pos < kc) emit(pos, half ? chl[1] : chl[0], half ? xs[1] : xs[0]);
+    };
+    // Team j ranks the first 64 candidates on its wave j and the rest on the next wave: waves w and w + 4 of a
+    // workgroup share a SIMD, so the ranking waves of the four teams sit on different SIMDs (four ranking waves on one
+    // SIMD took 2.2x as long).
+    auto rank_on_team = [&](uint32_t n) {
+        const uint32_t w0 = team & (kSelWaves - 1u), w1 = (team + 1u) & (kSelWaves - 1u);
+        if (tw == w0) rank_candidates(n, 0u);
+        else if (T::kRank > 64u && tw == w1 && n > 64u) rank_candidates(n, 1u);
     };
     if (scanner) {
         uint32_t xr[C];
@@ -419,10 +449,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
     }
     const u32x2 hd = *(const u32x2*)hdr;                    // state, candidates
     dec_stamp(p, blockIdx.x, 6);
-    // Team j ranks on its wave j: waves w and w + 4 of a workgroup share a SIMD, so the ranking waves of the four
-    // teams sit on four different SIMDs (four ranking waves on one SIMD took 2.2x as long).
-    const bool ranker = tw == (team & (kSelWaves - 1u));
-    if (hd[0] == kTeamFast && ranker) rank_candidates(hd[1]);
+    if (hd[0] == kTeamFast) rank_on_team(hd[1]);
     if (T::kSplit && any_split) {                          // uniform for the workgroup
         if (hd[0] == kTeamSplit) {                         // uniform per team
             const DecWindow w = dec_read_window<NW>(wc, lane, tw, kc);
@@ -454,7 +481,7 @@ __device__ __forceinline__ void dec_select_round(const DecParams& p, uint32_t cg
             if (ttid == 0) hdr[1] = n_sure;
         }
         __syncthreads();
-        if (hd[0] == kTeamSplit && ranker) rank_candidates(hdr[1]);
+        if (hd[0] == kTeamSplit) rank_on_team(hdr[1]);
     }
     dec_stamp(p, blockIdx.x, 7);
     if (any_general) {                                     // uniform for the workgroup; rare

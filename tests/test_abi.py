@@ -90,7 +90,7 @@ def test_dec_launch_plan_covers_the_layer(waves):
                     cpb, spb = -(-chunks // cg), -(-nseg // sg)
                     assert info.hip_slots_per_block >= cpb * k_chunk and info.hip_slots_per_block % 2 == 0
                     teams = 4 if waves == 16 else waves // 2
-                    red = max(waves * 2048, teams * (36 + 4 + 2 * 64 + 4) * 4)
+                    red = max(waves * 2048, teams * (36 + 4 + 2 * 128 + 4) * 4)
                     assert info.hip_lds_bytes == info.hip_slots_per_block * 8 + 4096 + red <= 60 * 1024
                     budget = n_tb * (16 // waves)
                     assert cg * sg <= budget or cg == 1 or chunks > budget, (K, N, n_tb, k_chunk, cg, sg)
