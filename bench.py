@@ -180,6 +180,55 @@ def link_leg(torch, full=False):
     return out
 
 
+def trace_leg(torch, ext, F, k_chunks=(8, 32), n_tb=32):
+    """Where a DEC-only launch spends its time: the role's own cycle stamps (library option `dec_trace`), median over
+    the workgroups of the last of five launches, in microseconds at the shader clock the stamps are taken with
+    (assumed 2.4 GHz).  Phases: activations (kernel start to the scanning teams' activations in registers), window
+    (scan, two barriers, compaction of the winning window), ranking (to the last selected channel written), fetch (the
+    residual rows over the host link), merge (cross-wave sum, scale, atomic adds); workgroup = start to end of a
+    workgroup (the counters of different dies are not synchronised, so stamps of different workgroups are never
+    compared)."""
+    import ctypes
+    import numpy as np
+    from decdec_amd import _lib
+    lib = _lib.load()
+    ghz = 2.4
+    g = torch.Generator().manual_seed(1)
+    out_rows = []
+    _lib.set_option("dec_trace", 1)
+    try:
+        for K, N in [(4096, 4096), (4096, 14336), (14336, 4096), (8192, 28672)]:
+            for kc in k_chunks:
+                rows = torch.zeros(K, dtype=torch.int32, device="cuda")
+                acts = torch.zeros(K, dtype=torch.float16, device="cuda")
+                th = F.calibrate_thresholds(K, g, draws=8)
+                x = F.make_activation(K, g).cuda()
+                cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), dtype=torch.int32)
+                out = torch.zeros(1, 1, N, device="cuda", dtype=torch.float16)
+                ctx = ext.create_dec_context(n_tb, rows, acts)
+                cfg = ext.create_dec_config(ctx, kc, cheat, torch.rand(N).half(), th)
+                info = ext.read_dec_config(cfg, native=True)
+                nb = info["hip_dec_blocks"]
+                buf = (ctypes.c_uint64 * (8 * nb))()
+                for _ in range(5):
+                    ext.dec(cfg, x, out)
+                    _lib.check(lib.decdec_debug_read_trace(buf, nb))
+                a = np.array(buf, dtype=np.uint64).reshape(nb, 8).astype(np.int64)
+                med = lambda v: round(float(np.median(v)) / ghz / 1e3, 2)
+                out_rows.append({"K": K, "N": N, "k_chunk": kc, "workgroups": nb, "chunk_groups": info["hip_chunk_groups"],
+                                 "segment_groups": info["hip_segment_groups"],
+                                 "activations_us": med(a[:, 5] - a[:, 0]), "window_us": med(a[:, 6] - a[:, 5]),
+                                 "ranking_us": med(a[:, 1] - a[:, 6]), "fetch_us": med(a[:, 2] - a[:, 1]),
+                                 "merge_us": med(a[:, 4] - a[:, 2]),
+                                 "workgroup_us": med(a[:, 4] - a[:, 0]),
+                                 "longest_workgroup_us": round(float((a[:, 4] - a[:, 0]).max()) / ghz / 1e3, 2)})
+                ext.destroy_dec_config(cfg)
+                ext.destroy_dec_context(ctx)
+    finally:
+        _lib.set_option("dec_trace", 0)
+    return out_rows
+
+
 def roofline_leg(torch, ext, protos, iters=240, calibrate_copy=False):
     """Average duration of the any-precision GEMV kernel on the 4096 -> 14336 shape, HIP events on the
     stream the kernel is launched on, rotating over private weight copies so each launch reads HBM."""
@@ -518,11 +567,12 @@ def main():
     ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers", "link"], default="all",
+    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers", "link", "trace"], default="all",
                     help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
                          "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 32); "
                          "helpers: the decode harness's helper kernels (output head, attention, norm, activation); "
-                         "link: zero-copy reads of pinned host memory over workgroup counts and request widths")
+                         "link: zero-copy reads of pinned host memory over workgroup counts and request widths; "
+                         "trace: phase timings of DEC-only launches from the role's own cycle stamps")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus N with N > 1 is not part of this build", file=sys.stderr)
@@ -542,6 +592,9 @@ def main():
         return
     if args.leg == "kernels":
         print(json.dumps({"kernels": kernels_leg(torch, ext, F)}))
+        return
+    if args.leg == "trace":
+        print(json.dumps({"dec_trace": trace_leg(torch, ext, F)}))
         return
     if args.leg == "roofline":
         _, _, protos, _ = build_layer_set(torch, F, 0, args.k_chunk, seed=0)

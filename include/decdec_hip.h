@@ -235,8 +235,9 @@ int decdec_greedy_pick(const void* logits, uint32_t n, int dtype, void* workspac
                        void* stream);
 
 /* Diagnostics: with option "dec_trace" = 1 every DEC workgroup stores shader-clock stamps of its
- * phases (0 start, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a
- * library-owned device buffer; this copies the first `workgroups` x 8 stamps to the host (it
+ * phases (0 start, 5 the scanning teams' activations in registers, 6 winning window compacted, 7 selected
+ * channels ranked, 1 selection done, 2 residual rows accumulated, 3 merged, 4 end) into a
+ * library-owned device buffer (at most 4096 workgroups); this copies the first `workgroups` x 8 stamps to the host (it
  * synchronises the device).  No counterpart in the reference. */
 int decdec_debug_read_trace(uint64_t* stamps_out, int workgroups);
 /* Diagnostics: a plain read kernel, nothing but loads -- the rate a fetch can reach on the memory `src` points at
