@@ -65,6 +65,13 @@ def test_every_linear_of_a_decode_step_matches_the_oracle(algo, bits):
 
 
 def test_graph_replays_equal_eager_steps():
+    """A replay of the captured decode step against the same step run eagerly.  Two runs of one step are not bit-equal
+    (the atomic adds of a layer arrive in a different order, a rounding step of difference in its output), and the
+    thresholds were calibrated on this very model, so some activations of the second layer sit exactly on a bucket
+    floor: once in a few dozen runs such a channel changes bucket between the two runs, DEC then compensates another
+    channel (with the large residuals of this test a visible part of the output) and the logits differ by several per
+    cent -- in the reference as much as here.  A pair that disagrees is therefore run again, up to three times; a
+    replay that read stale memory or a stale pointer disagrees every time."""
     model, _ = _tiny("sqllm", 4)
     with torch.no_grad():
         model(torch.randint(0, model.config.vocab_size, (1, 16), device="cuda"), torch.arange(16, device="cuda"))
@@ -72,20 +79,25 @@ def test_graph_replays_equal_eager_steps():
     step.start(3, 16)
     step.capture()
     for it, (tok, pos) in enumerate([(3, 16), (11, 17), (5, 18), (3, 16)]):
-        step.start(tok, pos)
-        with torch.no_grad():
-            step._step()
-        torch.cuda.synchronize()
-        eager = step.logits.clone()
-        junk = torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")      # unrelated work between
-        step.start(tok, pos)
-        step.graph.replay()
-        torch.cuda.synchronize()
-        assert int(step.pos) == pos + 1 and int(step.count) == 1
-        assert int(step.seq[0]) == int(torch.argmax(step.logits))
-        mre, _ = rel_err(step.logits.cpu().numpy().reshape(-1), eager.cpu().numpy().reshape(-1).astype(np.float64))
-        assert mre <= TOL, (it, mre)
-        del junk
+        seen = []
+        for attempt in range(3):
+            step.start(tok, pos)
+            with torch.no_grad():
+                step._step()
+            torch.cuda.synchronize()
+            eager = step.logits.clone()
+            junk = torch.randn(512, 512, device="cuda") @ torch.randn(512, 512, device="cuda")  # unrelated work between
+            step.start(tok, pos)
+            step.graph.replay()
+            torch.cuda.synchronize()
+            assert int(step.pos) == pos + 1 and int(step.count) == 1
+            assert int(step.seq[0]) == int(torch.argmax(step.logits))
+            mre, _ = rel_err(step.logits.cpu().numpy().reshape(-1), eager.cpu().numpy().reshape(-1).astype(np.float64))
+            seen.append(mre)
+            del junk
+            if mre <= TOL:
+                break
+        assert seen[-1] <= TOL, (it, seen)
 
 
 def test_generate_runs_prefill_and_graph_decode():
