@@ -59,6 +59,7 @@ def test_dec_and_fused_forms_on_random_shapes(seed, c_oracle):
         assert np.array_equal(got[filled], want_rows[filled]) and (got[~filled] == -7).all(), what
         want = base + c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows[filled], dt)
         mre, mae = rel_err(np_of(out).reshape(-1), want)
+        print(f"{what}: max rel err {mre:.3e} (bound {TOL[dt]:.0e}), mean abs err {mae:.3e}")
         assert mre <= TOL[dt], what + (mre, mae)
         ext.destroy_dec_config(cfg)
         ext.destroy_dec_context(ctx)
@@ -99,4 +100,5 @@ def test_base_gemvs_on_random_shapes(seed, c_oracle):
             want = c_oracle.lutgemm_gemv(np_of(x), qw.numpy(), np_of(alpha), np_of(qb), bits, group, dt)
         torch.cuda.synchronize()
         mre, mae = rel_err(np_of(out).reshape(-1), want)
+        print(f"{(seed, case, kind, K, N, bits, dt)}: max rel err {mre:.3e} (bound {TOL[dt]:.0e}), mean abs err {mae:.3e}")
         assert mre <= TOL[dt], (seed, case, kind, K, N, bits, dt, mre, mae)
