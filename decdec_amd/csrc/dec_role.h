@@ -1,5 +1,5 @@
 // DEC role: bucket top-k channel selection + zero-copy fetch of the selected 4-bit residual rows +
-// residual GEMV + atomic merge into the output.  One workgroup of 1024 threads (16 wave64) plays
+// residual GEMV + atomic merge into the output.  One workgroup of 16 wave64 (8 or 4 in the small forms) plays
 // this role; it is used by the standalone DEC kernels and, next to a base-GEMV role, by the fused
 // single-launch kernels.
 //
