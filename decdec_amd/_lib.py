@@ -48,6 +48,10 @@ SIGNATURES = {
     "decdec_dec_anyprec_batch": [_u32, ctypes.POINTER(_u64), _vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
                                  ctypes.POINTER(_vp), _i32, _i32, _u32, ctypes.POINTER(_u32), _vp],
     "decdec_dec_lutgemm": [_u64, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _u32, _u32, _vp],
+    "decdec_dec_lutgemm_batch": [_u32, ctypes.POINTER(_u64), _vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                                 ctypes.POINTER(_vp), ctypes.POINTER(_vp), _i32, _i32, _i32, _u32, ctypes.POINTER(_u32), _vp],
+    "decdec_dec_sqllm_batch": [_u32, ctypes.POINTER(_u64), _vp, ctypes.POINTER(_vp), ctypes.POINTER(_vp),
+                               ctypes.POINTER(_vp), _i32, _i32, _u32, ctypes.POINTER(_u32), _vp],
     "decdec_dec_sqllm": [_u64, _vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _vp],
     "decdec_dummy_anyprec": [_vp, _vp, _vp, _vp, _i32, _i32, _u32, _u32, _i32, _i64, _vp],
     "decdec_dummy_lutgemm": [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _u32, _u32, _i32, _i64, _vp],

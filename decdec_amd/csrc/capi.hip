@@ -1093,6 +1093,113 @@ int decdec_dec_sqllm(uint64_t h, const void* input, void* output, const void* ma
     return two_stream(c, &dp, have_dec, dtype, s, [&](hipStream_t sub) { return launch_sqllm(dtype, pl.p, pl.d, sub); });
 }
 
+// Batches of LUT-GEMM / SqueezeLLM layers on one input (the any-precision batch above, for the other two formats).
+// `plan(i, &params, &dims)` plans layer i's GEMV role for a 1024-thread workgroup, `single(i, have_config)` runs layer i
+// alone (the path without a batched kernel: fusion off, fp32).
+extern "C++" {
+template <typename GemvParams, typename Plan, typename Single, typename Launch>
+int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs, int dtype, uint32_t K,
+                 const uint32_t* out_features, GemvKind kind, double bytes_per_weight, bool batched_kernel,
+                 Plan plan, Single single, Launch launch) {
+    DD_CHECK(n >= 1 && n <= (uint32_t)kMaxBatch, "a batch holds 1 to %d layers, got %u", kMaxBatch, n);
+    DD_CHECK(outputs && out_features, "null pointer argument");
+    DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
+    for (uint32_t i = 0; i < n; ++i)
+        for (uint32_t j = 0; j < i; ++j)
+            DD_CHECK(outputs[i] != outputs[j], "the layers of a batch must have distinct outputs");
+    if (!g_opt.fusion || !batched_kernel) {
+        for (uint32_t i = 0; i < n; ++i) {
+            const int rc = single(i, configs != nullptr && configs[i] != 0);
+            if (rc != kOk) return rc;
+        }
+        return kOk;
+    }
+    BatchParams<GemvParams> b;
+    memset(&b, 0, sizeof(b));
+    b.n = n;
+    LaunchDims d{0, 1024u, 0};
+    uint32_t dec_total = 0, gemv_total = 0;
+    double dec_us = 0.0, weight_bytes = 0.0;
+    bool any_dec = false;
+    for (uint32_t i = 0; i < n; ++i) {
+        Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
+        bool have_dec = false;
+        if (configs && configs[i]) {
+            int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
+            if (rc != kOk) return rc;
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i]) == 0;
+            b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
+        }
+        LaunchDims ld{0, 0, 0};
+        int rc = plan(i, &b.gp[i], &ld);
+        if (rc != kOk) return rc;
+        DD_CHECK(ld.block == 1024u, "internal: batched layers need 1024-thread workgroups");
+        d.lds = std::max(d.lds, ld.lds);
+        if (have_dec) {
+            dec_total += c->plans[2].cg * c->plans[2].sg;
+            d.lds = std::max(d.lds, c->plans[2].lds);
+            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
+            any_dec = true;
+        }
+        gemv_total += ld.grid;
+        weight_bytes += bytes_per_weight * out_features[i] * K;
+        b.dec_end[i] = dec_total;
+        b.gemv_end[i] = gemv_total;
+    }
+    for (uint32_t i = n; i < (uint32_t)kMaxBatch; ++i) { b.dec_end[i] = dec_total; b.gemv_end[i] = gemv_total; }
+    d.grid = dec_total + gemv_total;
+    const double flip = kind == kSqllm ? 1.15 : 1.3;      // the single-layer rule (fused_two_per_cu) applied to the batch
+    if (g_opt.fused_two_per_cu >= 0) d.two_per_cu = g_opt.fused_two_per_cu != 0;
+    else d.two_per_cu = !any_dec || (8.0 + dec_us) < flip * gemv_estimate_us(kind, weight_bytes);
+    DD_HIP(launch(b, d));
+    return kOk;
+}
+}  // extern "C++"
+
+int decdec_dec_lutgemm_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                             const void* const* q_weights, const void* const* alphas, const void* const* q_biases,
+                             int bits, int group_size, int dtype, uint32_t K, const uint32_t* out_features, void* stream) {
+    DD_CHECK(q_weights && alphas && q_biases, "null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    return batch_common<LutgemmParams>(
+        n, configs, input, outputs, dtype, K, out_features, kLutgemm, bits / 8.0, dtype != DECDEC_FP32,
+        [&](uint32_t i, LutgemmParams* gp, LaunchDims* ld) {
+            LutgemmPlan pl;
+            const int rc = plan_lutgemm(input, outputs[i], q_weights[i], alphas[i], q_biases[i], bits, group_size, dtype, K,
+                                        out_features[i], true, &pl);
+            *gp = pl.p; *ld = pl.d;
+            return rc;
+        },
+        [&](uint32_t i, bool have_config) {
+            return have_config ? decdec_dec_lutgemm(configs[i], input, outputs[i], q_weights[i], alphas[i], q_biases[i], bits,
+                                                    group_size, dtype, K, out_features[i], stream)
+                               : decdec_lutgemm_gemv(input, outputs[i], q_weights[i], alphas[i], q_biases[i], bits, group_size,
+                                                     dtype, K, out_features[i], stream);
+        },
+        [&](const BatchParams<LutgemmParams>& b, const LaunchDims& d) { return launch_dec_lutgemm_batch(dtype, b, d, s); });
+}
+
+int decdec_dec_sqllm_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                           const void* const* qweights, const void* const* luts, int bits, int dtype, uint32_t K,
+                           const uint32_t* out_features, void* stream) {
+    DD_CHECK(qweights && luts, "null pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    return batch_common<SqllmParams>(
+        n, configs, input, outputs, dtype, K, out_features, kSqllm, bits / 8.0, dtype != DECDEC_FP32,
+        [&](uint32_t i, SqllmParams* gp, LaunchDims* ld) {
+            SqllmPlan pl;
+            const int rc = plan_sqllm(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], true, &pl);
+            *gp = pl.p; *ld = pl.d;
+            return rc;
+        },
+        [&](uint32_t i, bool have_config) {
+            return have_config ? decdec_dec_sqllm(configs[i], input, outputs[i], qweights[i], luts[i], bits, dtype, K,
+                                                  out_features[i], stream)
+                               : decdec_sqllm_gemv(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], stream);
+        },
+        [&](const BatchParams<SqllmParams>& b, const LaunchDims& d) { return launch_dec_sqllm_batch(dtype, b, d, s); });
+}
+
 // ---------------------------------------------------------------- dummies
 int decdec_dummy_anyprec(const void* input, void* output, const void* qweight, const void* lut, int bits,
                          int dtype, uint32_t K, uint32_t N, int dummy_cu, int64_t iters, void* stream) {

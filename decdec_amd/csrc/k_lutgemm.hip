@@ -17,6 +17,22 @@ __global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_lutgemm_kernel(co
     else lutgemm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
 }
 
+// Up to kMaxBatch layers on one input in one launch: a workgroup finds its layer and plays the DEC or the GEMV role
+// for it, exactly as in the single-layer kernel above.
+template <int DT, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_lutgemm_batch_kernel(const BatchParams<LutgemmParams> b) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t ndec = b.dec_end[kMaxBatch - 1];
+    uint32_t layer, local;
+    if (blockIdx.x < ndec) {
+        batch_locate(b.dec_end, blockIdx.x, layer, local);
+        dec_role<DT>(b.dp[layer], local, smem);
+    } else {
+        batch_locate(b.gemv_end, blockIdx.x - ndec, layer, local);
+        lutgemm_role<DT>(b.gp[layer], local, smem);
+    }
+}
+
 hipError_t launch_lutgemm(int dt, const LutgemmParams& p, const LaunchDims& d, hipStream_t s) {
     switch (dt) {
         case kFP32: hipLaunchKernelGGL(lutgemm_kernel<kFP32>, dim3(d.grid), dim3(d.block), d.lds, s, p); break;
@@ -45,6 +61,19 @@ hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
             else hipLaunchKernelGGL((dec_lutgemm_kernel<kBF16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
             break;
         default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_lutgemm_batch(int dt, const BatchParams<LutgemmParams>& b, const LaunchDims& d, hipStream_t s) {
+    const dim3 grid(d.grid), block(d.block);
+    if ((dt != kFP16 && dt != kBF16) || d.block != 1024u) return hipErrorInvalidValue;
+    if (d.two_per_cu) {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_lutgemm_batch_kernel<kFP16, true>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_lutgemm_batch_kernel<kBF16, true>), grid, block, d.lds, s, b);
+    } else {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_lutgemm_batch_kernel<kFP16, false>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_lutgemm_batch_kernel<kBF16, false>), grid, block, d.lds, s, b);
     }
     return hipGetLastError();
 }

@@ -17,6 +17,22 @@ __global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_sqllm_kernel(cons
     else sqllm_role<DT>(gp, blockIdx.x - dec_blocks, smem);
 }
 
+// Up to kMaxBatch layers on one input in one launch: a workgroup finds its layer and plays the DEC or the GEMV role
+// for it, exactly as in the single-layer kernel above.
+template <int DT, bool TWO>
+__global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_sqllm_batch_kernel(const BatchParams<SqllmParams> b) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t ndec = b.dec_end[kMaxBatch - 1];
+    uint32_t layer, local;
+    if (blockIdx.x < ndec) {
+        batch_locate(b.dec_end, blockIdx.x, layer, local);
+        dec_role<DT>(b.dp[layer], local, smem);
+    } else {
+        batch_locate(b.gemv_end, blockIdx.x - ndec, layer, local);
+        sqllm_role<DT>(b.gp[layer], local, smem);
+    }
+}
+
 // The 4-bit pair table needs more than the 64 KB of dynamic LDS a kernel gets by default.
 template <typename K>
 static hipError_t allow_large_lds(K kernel) {
@@ -30,6 +46,8 @@ static hipError_t sqllm_prepare() {
         acc(allow_large_lds(dec_sqllm_kernel<kFP32, false>));
         acc(allow_large_lds(dec_sqllm_kernel<kFP16, false>)); acc(allow_large_lds(dec_sqllm_kernel<kFP16, true>));
         acc(allow_large_lds(dec_sqllm_kernel<kBF16, false>)); acc(allow_large_lds(dec_sqllm_kernel<kBF16, true>));
+        acc(allow_large_lds(dec_sqllm_batch_kernel<kFP16, false>)); acc(allow_large_lds(dec_sqllm_batch_kernel<kFP16, true>));
+        acc(allow_large_lds(dec_sqllm_batch_kernel<kBF16, false>)); acc(allow_large_lds(dec_sqllm_batch_kernel<kBF16, true>));
         return e;
     }();
     return done;
@@ -62,6 +80,20 @@ hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
             else hipLaunchKernelGGL((dec_sqllm_kernel<kBF16, false>), grid, block, d.lds, s, dp, dec_blocks, gp);
             break;
         default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dec_sqllm_batch(int dt, const BatchParams<SqllmParams>& b, const LaunchDims& d, hipStream_t s) {
+    if (hipError_t e = sqllm_prepare(); e != hipSuccess) return e;
+    const dim3 grid(d.grid), block(d.block);
+    if ((dt != kFP16 && dt != kBF16) || d.block != 1024u) return hipErrorInvalidValue;
+    if (d.two_per_cu) {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_sqllm_batch_kernel<kFP16, true>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_sqllm_batch_kernel<kBF16, true>), grid, block, d.lds, s, b);
+    } else {
+        if (dt == kFP16) hipLaunchKernelGGL((dec_sqllm_batch_kernel<kFP16, false>), grid, block, d.lds, s, b);
+        else hipLaunchKernelGGL((dec_sqllm_batch_kernel<kBF16, false>), grid, block, d.lds, s, b);
     }
     return hipGetLastError();
 }

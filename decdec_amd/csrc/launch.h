@@ -67,6 +67,9 @@ hipError_t launch_dec_lutgemm(int dt, const DecParams& dp, uint32_t dec_blocks,
                               const LutgemmParams& gp, const LaunchDims& d, hipStream_t s);
 hipError_t launch_dec_sqllm(int dt, const DecParams& dp, uint32_t dec_blocks,
                             const SqllmParams& gp, const LaunchDims& d, hipStream_t s);
+// Batches of up to kMaxBatch LUT-GEMM / SqueezeLLM layers on one input (16-bit types), as launch_dec_anyprec_batch.
+hipError_t launch_dec_lutgemm_batch(int dt, const BatchParams<LutgemmParams>& b, const LaunchDims& d, hipStream_t s);
+hipError_t launch_dec_sqllm_batch(int dt, const BatchParams<SqllmParams>& b, const LaunchDims& d, hipStream_t s);
 
 // Decode-step helpers (k_decode.hip).  `pos` points at the token position in device memory.
 struct RopeCacheParams {

@@ -361,6 +361,44 @@ def dec_sqllm(dec_config: int, input, output, q_weight, lut, bitwidth: int) -> N
                                             int(bitwidth), _dt(input), input.size(2), output.size(2), _stream()))
 
 
+def _batch_arrays(dec_configs, input, outputs, per_layer):
+    n = len(outputs)
+    _check(1 <= n <= 4 and all(len(seq) == n for seq in per_layer), "a batch holds 1 to 4 layers")
+    cfgs = [int(c) if c else 0 for c in (dec_configs if dec_configs is not None else [0] * n)]
+    _check(len(cfgs) == n, "one config (or 0) per layer")
+    for c, out in zip(cfgs, outputs):
+        if c:
+            _check_dec_io(c, input, out)
+    arr_c = (ctypes.c_uint64 * n)(*cfgs)
+    arr_o = (ctypes.c_void_p * n)(*[_ptr(t) for t in outputs])
+    arrs = [(ctypes.c_void_p * n)(*[_ptr(t) for t in seq]) for seq in per_layer]
+    arr_n = (ctypes.c_uint32 * n)(*[t.size(2) for t in outputs])
+    return n, arr_c, arr_o, arrs, arr_n
+
+
+def dec_lutgemm_batch(dec_configs, input, outputs, q_weights, alphas, q_biases, bitwidth: int, group_size: int) -> None:
+    """Layers that read the same `input`, in one launch: layer i is dec_lutgemm(dec_configs[i], input, outputs[i],
+    q_weights[i], alphas[i], q_biases[i], bitwidth, group_size), or lutgemm_gemv when dec_configs[i] is 0 / None.
+    Not in the reference."""
+    _check(input.dtype in _DT, "Unsupported data type.")
+    n, arr_c, arr_o, (arr_q, arr_a, arr_b), arr_n = _batch_arrays(dec_configs, input, outputs, (q_weights, alphas, q_biases))
+    for out, qw, al, qb in zip(outputs, q_weights, alphas, q_biases):
+        _check_lutgemm(input, out, qw, al, qb, bitwidth, group_size)
+    _lib.check(_lib.load().decdec_dec_lutgemm_batch(n, arr_c, _ptr(input), arr_o, arr_q, arr_a, arr_b, int(bitwidth),
+                                                    int(group_size), _dt(input), input.size(2), arr_n, _stream()))
+
+
+def dec_sqllm_batch(dec_configs, input, outputs, q_weights, luts, bitwidth: int) -> None:
+    """Layers that read the same `input`, in one launch: layer i is dec_sqllm(dec_configs[i], input, outputs[i],
+    q_weights[i], luts[i], bitwidth), or sqllm_gemv when dec_configs[i] is 0 / None.  Not in the reference."""
+    _check(input.dtype in _DT, "Unsupported data type.")
+    n, arr_c, arr_o, (arr_q, arr_l), arr_n = _batch_arrays(dec_configs, input, outputs, (q_weights, luts))
+    for out, qw, lut in zip(outputs, q_weights, luts):
+        _check_sqllm(input, out, qw, lut, bitwidth)
+    _lib.check(_lib.load().decdec_dec_sqllm_batch(n, arr_c, _ptr(input), arr_o, arr_q, arr_l, int(bitwidth), _dt(input),
+                                                  input.size(2), arr_n, _stream()))
+
+
 def dummy_anyprec(input, output, qweight, lut, bitwidth: int, dummy_sm: int, dummy_iters: int) -> None:
     """decdec.cu:874-893."""
     _check(input.dtype in (torch.float16, torch.bfloat16), "dummy_anyprec supports FP16/BF16 only.")
@@ -395,4 +433,4 @@ REFERENCE_API = (
     "dec", "unfused_dec", "anyprec_dequant", "anyprec_gemv", "lutgemm_gemv", "sqllm_gemv",
     "dec_anyprec", "dec_lutgemm", "dec_sqllm", "dummy_anyprec", "dummy_lutgemm", "dummy_sqllm",
 )
-__all__ = list(REFERENCE_API) + ["destroy_dec_context", "dec_anyprec_batch"]
+__all__ = list(REFERENCE_API) + ["destroy_dec_context", "dec_anyprec_batch", "dec_lutgemm_batch", "dec_sqllm_batch"]

@@ -167,6 +167,17 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
                              const void* const* qweights, const void* const* luts, int bitwidth, int dtype,
                              uint32_t in_features, const uint32_t* out_features, void* stream);
 
+/* The same for LUT-GEMM and SqueezeLLM layers (argument meaning as in decdec_dec_lutgemm / decdec_dec_sqllm, one
+ * pointer per layer; fp16 and bf16 run in one launch, fp32 as one call per layer with the same result).  No
+ * counterpart in the reference. */
+int decdec_dec_lutgemm_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                             const void* const* q_weights, const void* const* alphas, const void* const* q_biases,
+                             int bitwidth, int group_size, int dtype, uint32_t in_features,
+                             const uint32_t* out_features, void* stream);
+int decdec_dec_sqllm_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
+                           const void* const* qweights, const void* const* luts, int bitwidth, int dtype,
+                           uint32_t in_features, const uint32_t* out_features, void* stream);
+
 /* Decode-step helpers for a caller that drives the linear layers from a captured decode step (the
  * reference leaves these operations to torch.compile, end-to-end/generate.py; they have no counterpart in
  * its extension).  All tensors are fp16 or bf16 in device memory; `pos_device` points at the token position

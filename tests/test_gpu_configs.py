@@ -272,6 +272,65 @@ def test_batched_layers_match_the_oracle_layer_by_layer(dt, bits, c_oracle):
         ext.destroy_dec_config(l["cfg"])
 
 
+@pytest.mark.parametrize("kind,dt", [("lutgemm", "fp16"), ("lutgemm", "bf16"), ("lutgemm", "fp32"),
+                                     ("sqllm", "fp16"), ("sqllm", "bf16"), ("sqllm", "fp32")])
+def test_batched_lutgemm_and_sqllm_layers_match_the_oracle(kind, dt, c_oracle):
+    """dec_lutgemm_batch / dec_sqllm_batch: three layers on one input in one launch (fp32: the per-layer path), DEC on
+    all, on the middle one only, on none; every output against the oracle, every context's selection bit-exact."""
+    from tests.helpers import TORCH_DT
+    dtype = TORCH_DT[dt]
+    K, Ns, k_chunk, group = 4096, (2048, 1024, 520), 32, 128
+    bits = 3 if kind == "lutgemm" else 4
+    g = torch.Generator().manual_seed(11)
+    x = F.make_activation(K, g, dtype=dtype)
+    xn = np_of(x)
+    layers = []
+    for N in Ns:
+        W = (torch.randn(N, K, generator=g) * 0.02).half()
+        cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32)
+        scales = (torch.rand(N, generator=g) * 1e-3 + 5e-4).to(dtype)
+        th = F.calibrate_thresholds(K, g, draws=8, dtype=dtype)
+        ctx, rows, acts = _ctx(16, K, dtype)
+        cfg = ext.create_dec_config(ctx, k_chunk, cheat, scales, th)
+        if kind == "lutgemm":
+            q, s, z = F.awq_pseudo_quantize(W, bits, group)
+            qw, alpha, q_bias = F.pack_bcq(q, s, z, bits, dtype=dtype)
+            weights = (qw, alpha, q_bias)
+            base = c_oracle.lutgemm_gemv(xn, qw.numpy(), np_of(alpha), np_of(q_bias), bits, group, dt)
+        else:
+            idx, lut = F.quantize_uniform_rows(W, bits)
+            mat, lut = F.pack_sqllm(idx, bits), lut.to(dtype)
+            weights = (mat, lut)
+            base = c_oracle.sqllm_gemv(xn, mat.numpy(), np_of(lut), bits, dt)
+        layers.append(dict(N=N, weights=[w.cuda() for w in weights], cheat=cheat, scales=scales, th=th, cfg=cfg, rows=rows,
+                           acts=acts, base=base))
+    xc = x.cuda()
+    per_layer = list(zip(*[l["weights"] for l in layers]))             # one sequence per weight kind
+    for mode in ("all", "middle", "none"):
+        outs = [torch.zeros(1, 1, l["N"], dtype=dtype, device="cuda") for l in layers]
+        for l in layers:
+            l["rows"].fill_(-7)
+        cfgs = {"all": [l["cfg"] for l in layers], "middle": [0, layers[1]["cfg"], None], "none": None}[mode]
+        if kind == "lutgemm":
+            ext.dec_lutgemm_batch(cfgs, xc, outs, *per_layer, bits, group)
+        else:
+            ext.dec_sqllm_batch(cfgs, xc, outs, *per_layer, bits)
+        torch.cuda.synchronize()
+        for li, l in enumerate(layers):
+            with_dec = cfgs is not None and bool(cfgs[li])
+            want = l["base"]
+            if with_dec:
+                want_rows, _, _ = O.select_channels(xn, np_of(l["th"]), k_chunk, dt)
+                k = k_chunk * K // 1024
+                assert np.array_equal(l["rows"].cpu().numpy()[:k], want_rows[:k]), (mode, li)
+                want = want + c_oracle.dec_apply(xn, l["cheat"].numpy(), np_of(l["scales"]), want_rows[:k], dt)
+            else:
+                assert (l["rows"].cpu().numpy() == -7).all(), (mode, li)
+            check_output(np_of(outs[li]).reshape(-1), want, dt, (kind, mode, li))
+    for l in layers:
+        ext.destroy_dec_config(l["cfg"])
+
+
 # --------------------------------------------------------------------------------------------------
 # Phi-3-medium: LUT-GEMM 3-bit, group 128, with DEC
 # --------------------------------------------------------------------------------------------------
