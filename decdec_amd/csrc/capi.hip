@@ -443,7 +443,8 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
 struct LutgemmPlan { LutgemmParams p; LaunchDims d; };
 
 int plan_lutgemm(const void* input, void* output, const void* qw, const void* alpha, const void* q_bias, int bits,
-                 int group_size, int dtype, uint32_t K, uint32_t N, bool fused_block, LutgemmPlan* pl) {
+                 int group_size, int dtype, uint32_t K, uint32_t N, bool fused_block, LutgemmPlan* pl,
+                 uint32_t slots_avail = 0) {
     DD_CHECK(bits >= 1 && bits <= 8, "Bitwidth must be between 1 and 8.");
     DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
     DD_CHECK(input && output && qw && alpha && q_bias, "null pointer argument");
@@ -470,7 +471,8 @@ int plan_lutgemm(const void* input, void* output, const void* qw, const void* al
         p.slice_tiles = std::max(1u, std::min(4u, cdiv(tiles, kt * waves)));
         p.k_tiles = cdiv(tiles, p.slice_tiles * waves);
     } else {
-        const uint32_t slots = 2u * device_cus();
+        // workgroup slots this layer can count on: the whole device, or its share of it inside a batched launch
+        const uint32_t slots = slots_avail ? slots_avail : 2u * device_cus();
         uint32_t best_cost = ~0u;
         for (uint32_t kr = 1; kr <= 9; ++kr) {
             const uint32_t slice = cdiv(tiles, kr * waves);
@@ -1165,8 +1167,12 @@ int decdec_dec_lutgemm_batch(uint32_t n, const uint64_t* configs, const void* in
         n, configs, input, outputs, dtype, K, out_features, kLutgemm, bits / 8.0, dtype != DECDEC_FP32,
         [&](uint32_t i, LutgemmParams* gp, LaunchDims* ld) {
             LutgemmPlan pl;
+            // the layers of a batch share the device in proportion to their widths
+            uint64_t total = 0;
+            for (uint32_t j = 0; j < n; ++j) total += out_features[j];
+            const uint32_t share = (uint32_t)std::max<uint64_t>(32u, (uint64_t)2u * device_cus() * out_features[i] / std::max<uint64_t>(total, 1));
             const int rc = plan_lutgemm(input, outputs[i], q_weights[i], alphas[i], q_biases[i], bits, group_size, dtype, K,
-                                        out_features[i], true, &pl);
+                                        out_features[i], true, &pl, share);
             *gp = pl.p; *ld = pl.d;
             return rc;
         },
