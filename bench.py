@@ -717,6 +717,26 @@ def main():
     result["roofline_link"] = roofline_link_leg(torch, ext, protos, args.k_chunk, args.n_tb, link_leg(torch))
     drop_configs(ctxs, cfgs)
 
+    # The same step with every layer's residual resident in HBM (a private device copy per layer: 3.3 GB, which a
+    # 288 GB device holds beside the weights; the library uses a device residual in place).  Not the metric -- the
+    # metric's residuals live in host memory -- but what this machine can do with the same operator.
+    dev_ctxs = [ext.create_dec_context(args.n_tb, r, a) for r, a in scratch]
+    err_fd = os.dup(2)                                    # the library warns once per config that the residual is on the device
+    null_fd = os.open(os.devnull, os.O_WRONLY)
+    os.dup2(null_fd, 2)
+    try:
+        dev_cfgs = [ext.create_dec_config(dev_ctxs[BRANCH[l["name"]]], args.k_chunk, l["cheat"].cuda(), l["scales"], l["th"])
+                    for l in layers]
+    finally:
+        os.dup2(err_fd, 2)
+        os.close(null_fd)
+        os.close(err_fd)
+    cfgs = dev_cfgs
+    dev_us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), args.steps, args.warmup)
+    result["residual_in_hbm_us_per_token"] = round(dev_us * scale, 2)
+    result["residual_in_hbm_dec_slowdown_pct"] = round((dev_us / base_us - 1) * 100, 2)
+    drop_configs(dev_ctxs, dev_cfgs)
+
     if args.sweep:
         sweep = []
         for n_tb in (8, 16, 32, 64):
