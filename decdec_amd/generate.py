@@ -76,9 +76,11 @@ def calibrate_thresholds(model: Transformer, seq_len: int = 256, passes: int = 2
     return artifacts.collect_thresholds(named, run, dtype=model.dtype)
 
 
-def random_dec_data(model: Transformer, thresholds: dict, seed: int = 2, residual_scale: float = 2e-4) -> dict:
+def random_dec_data(model: Transformer, thresholds: dict, seed: int = 2, residual_scale: float = 2e-4,
+                    residual_device=None) -> dict:
     """Random 4-bit residual words and scales per module (one tensor per module shape, shared by the layers:
-    every config pins its own copy) with the given thresholds."""
+    every config pins its own copy) with the given thresholds.  With `residual_device` every layer gets a private
+    copy of its residual on that device instead (the library then reads it in place: residuals resident in HBM)."""
     gen = torch.Generator().manual_seed(seed)
     per_shape = {}
     out = {}
@@ -91,6 +93,8 @@ def random_dec_data(model: Transformer, thresholds: dict, seed: int = 2, residua
                 per_shape[(K, N)] = (q, s)
             q, s = per_shape[(K, N)]
             p = f"layers.{i}.{key}."
+            if residual_device is not None:
+                q = q.to(residual_device)                  # a new device tensor per layer
             out[p + "q_residual"], out[p + "scales"], out[p + "thresholds"] = q, s, thresholds[f"layers.{i}.{key}"]
     return out
 
@@ -210,6 +214,8 @@ def main(argv=None):
     ap.add_argument("--max-seq-length", type=int, default=2048)
     ap.add_argument("--n-layer", type=int, default=None, help="fewer layers than the named model (smoke runs)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--residual-on-device", action="store_true",
+                    help="keep every layer's residual in device memory instead of pinned host memory")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="library option (decdec_set_option), e.g. fusion=0; may be repeated")
     args = ap.parse_args(argv)
@@ -231,7 +237,7 @@ def main(argv=None):
     n = args.max_new_tokens - 1
     log(f"base: {n / t_base:.1f} tokens/s; calibrating thresholds")
     th = calibrate_thresholds(model)
-    model.load_dec_data(random_dec_data(model, th))
+    model.load_dec_data(random_dec_data(model, th, residual_device="cuda" if args.residual_on_device else None))
     k_max = max(max(ks) for ks in k_sets)
     model.create_dec_context(args.n_tb, buffer_size=max(1024, k_max * (model.config.intermediate_size // 1024 + 1)))
     for i, ks in enumerate(k_sets):
@@ -247,7 +253,8 @@ def main(argv=None):
             "prompt_len": args.prompt_len, "new_tokens": args.max_new_tokens, "graph": not args.no_graph,
             "tokens_per_s_base": round(n / t_base, 2), "tokens_per_s_dec": round(n / t_dec, 2),
             "ms_per_token_base": round(t_base / n * 1e3, 4), "ms_per_token_dec": round(t_dec / n * 1e3, 4),
-            "dec_slowdown_pct": round((t_dec / t_base - 1) * 100, 2), "data": "synthetic (random weights and prompt)"}),
+            "dec_slowdown_pct": round((t_dec / t_base - 1) * 100, 2), "data": "synthetic (random weights and prompt)",
+            "residual": "device memory" if args.residual_on_device else "pinned host memory"}),
             flush=True)
 
 
