@@ -331,6 +331,91 @@ def test_batched_lutgemm_and_sqllm_layers_match_the_oracle(kind, dt, c_oracle):
         ext.destroy_dec_config(l["cfg"])
 
 
+def _random_anyprec3(K, N, g):
+    """Random 3-bit planes and a sorted random LUT per row: everything the GEMV reads, without quantising a weight
+    matrix (a 70B-size layer is built in a second)."""
+    qweight = torch.randint(-2 ** 31, 2 ** 31 - 1, (3, N, K // 32), generator=g, dtype=torch.int64).to(torch.int32)
+    lut = (torch.randn(N, 8, generator=g) * 0.02).sort(dim=1).values.half()
+    return qweight.contiguous(), lut.contiguous()
+
+
+@pytest.mark.parametrize("two_per_cu", [0, 1])
+@pytest.mark.parametrize("Ns", [(14336, 14336), (4096, 1024, 1024)], ids=["gate_up", "q_k_v"])
+def test_batched_launch_at_the_benchmark_shapes(Ns, two_per_cu, c_oracle):
+    """dec_anyprec_batch as the benchmark launches it: gate | up = 2 x (4096 -> 14336) and q | k | v = 4096 -> (4096, 1024,
+    1024) at k_chunk 32, n_tb 32, with the fused kernel instance chosen both ways.  Every layer's selection bit-exact,
+    every output against the oracle; then the same batch with ONE context shared by all layers (the scratch read-back
+    then belongs to whichever layer wrote last, the outputs must still be right)."""
+    K, k_chunk, n_tb = 4096, 32, 32
+    g = torch.Generator().manual_seed(sum(Ns) + two_per_cu)
+    x = F.make_activation(K, g)
+    xn = np_of(x)
+    k = k_chunk * K // 1024
+    layers = []
+    for N in Ns:
+        qweight, lut = _random_anyprec3(K, N, g)
+        cheat = torch.randint(-2 ** 31, 2 ** 31 - 1, (K, N // 8), generator=g, dtype=torch.int64).to(torch.int32)
+        scales = (torch.rand(N, generator=g) * 1e-3 + 5e-4).half()
+        th = F.calibrate_thresholds(K, g, draws=8)
+        want_rows, _, _ = O.select_channels(xn, np_of(th), k_chunk)
+        want = c_oracle.anyprec_gemv(xn, qweight.numpy(), np_of(lut), 3) + \
+            c_oracle.dec_apply(xn, cheat.numpy(), np_of(scales), want_rows[:k])
+        layers.append(dict(N=N, qweight=qweight.cuda(), lut=lut.cuda(), cheat=cheat, scales=scales, th=th,
+                           want_rows=want_rows, want=want))
+    xc = x.cuda()
+    _lib.set_option("fused_two_per_cu", two_per_cu)
+    try:
+        own = [_ctx(n_tb, K) for _ in layers]
+        cfgs = [ext.create_dec_config(c[0], k_chunk, l["cheat"], l["scales"], l["th"]) for c, l in zip(own, layers)]
+        outs = [torch.zeros(1, 1, l["N"], dtype=torch.float16, device="cuda") for l in layers]
+        ext.dec_anyprec_batch(cfgs, xc, outs, [l["qweight"] for l in layers], [l["lut"] for l in layers], 3)
+        torch.cuda.synchronize()
+        for li, (l, c) in enumerate(zip(layers, own)):
+            assert np.array_equal(c[1].cpu().numpy()[:k], l["want_rows"][:k]), ("selection", li)
+            check_output(np_of(outs[li]).reshape(-1), l["want"], "fp16", ("own contexts", Ns, two_per_cu, li))
+        for cfg in cfgs:
+            ext.destroy_dec_config(cfg)
+        shared = _ctx(n_tb, K)
+        cfgs = [ext.create_dec_config(shared[0], k_chunk, l["cheat"], l["scales"], l["th"]) for l in layers]
+        outs = [torch.zeros(1, 1, l["N"], dtype=torch.float16, device="cuda") for l in layers]
+        ext.dec_anyprec_batch(cfgs, xc, outs, [l["qweight"] for l in layers], [l["lut"] for l in layers], 3)
+        torch.cuda.synchronize()
+        for li, l in enumerate(layers):
+            check_output(np_of(outs[li]).reshape(-1), l["want"], "fp16", ("one shared context", Ns, two_per_cu, li))
+        for cfg in cfgs:
+            ext.destroy_dec_config(cfg)
+    finally:
+        _lib.set_option("fused_two_per_cu", -1)
+
+
+@pytest.mark.parametrize("K,N", [(28672, 8192), (8192, 28672)])
+def test_anyprec_at_llama3_70b_gate_and_down(K, N, c_oracle):
+    """Any-precision 3-bit at the two large 70B linears (28672 -> 8192 is the 14-slice, 896-thread launch form):
+    the GEMV alone, then dec_anyprec at k_chunk 16 and 32, against the oracle; indices bit-exact."""
+    g = torch.Generator().manual_seed(K + N)
+    qweight, lut = _random_anyprec3(K, N, g)
+    L = _dec_only_layer(K, N, seed=K - N)
+    xn = np_of(L["x"])
+    xc, qc, lc = L["x"].cuda(), qweight.cuda(), lut.cuda()
+    base = c_oracle.anyprec_gemv(xn, qweight.numpy(), np_of(lut), 3)
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.anyprec_gemv(xc, out, qc, lc, 3)
+    torch.cuda.synchronize()
+    check_output(np_of(out).reshape(-1), base, "fp16", ("anyprec_gemv", K, N))
+    for k_chunk in (16, 32):
+        ctx, rows, acts = _ctx(32, K)
+        cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+        out.zero_()
+        ext.dec_anyprec(cfg, xc, out, qc, lc, 3)
+        torch.cuda.synchronize()
+        k = k_chunk * K // 1024
+        want_rows, _, _ = O.select_channels(xn, np_of(L["th"]), k_chunk)
+        assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k]), (K, N, k_chunk)
+        want = base + c_oracle.dec_apply(xn, L["cheat"].numpy(), np_of(L["scales"]), want_rows[:k])
+        check_output(np_of(out).reshape(-1), want, "fp16", ("dec_anyprec", K, N, k_chunk))
+        ext.destroy_dec_config(cfg)
+
+
 # --------------------------------------------------------------------------------------------------
 # Phi-3-medium: LUT-GEMM 3-bit, group 128, with DEC
 # --------------------------------------------------------------------------------------------------
@@ -357,6 +442,32 @@ def test_dec_lutgemm_at_phi3_shapes(K, N, c_oracle):
     base = c_oracle.lutgemm_gemv(xn, qw.numpy(), np_of(alpha), np_of(q_bias), bits, group)
     check_output(np_of(base_out).reshape(-1), base, "fp16", ("lutgemm_gemv", K, N))
     want = base + c_oracle.dec_apply(xn, L["cheat"].numpy(), np_of(L["scales"]), want_rows[:k])
+    check_output(np_of(out).reshape(-1), want, "fp16", ("dec_lutgemm", K, N))
+    ext.destroy_dec_config(cfg)
+
+
+def test_dec_lutgemm_at_phi3_gate_up(c_oracle):
+    """dec_lutgemm at Phi-3-medium's fused gate_up projection, 5120 -> 35840 (70 column segments of 512 outputs),
+    k_chunk 32: indices bit-exact and the output against the oracle.  Random packed BCQ words, scales and offsets
+    (what the kernel reads; no weight matrix is quantised), random residual words."""
+    K, N, k_chunk, bits, group = 5120, 35840, 32, 3, 128
+    g = torch.Generator().manual_seed(K + N)
+    qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 32, bits, N), generator=g, dtype=torch.int64).to(torch.int32)
+    alpha = (torch.rand(K // group, bits, N, generator=g) * 4e-3 + 1e-3).half()
+    q_bias = (torch.randn(K // group, N, generator=g) * 2e-3).half()
+    L = _dec_only_layer(K, N, seed=N - K)
+    ctx, rows, acts = _ctx(32, K)
+    cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+    out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+    ext.dec_lutgemm(cfg, L["x"].cuda(), out, qw.cuda(), alpha.cuda(), q_bias.cuda(), bits, group)
+    torch.cuda.synchronize()
+    xn = np_of(L["x"])
+    k = k_chunk * K // 1024
+    want_rows, want_acts, _ = O.select_channels(xn, np_of(L["th"]), k_chunk)
+    assert np.array_equal(rows.cpu().numpy()[:k], want_rows[:k])
+    assert np.array_equal(np_of(acts)[:k], want_acts[:k].astype(np.float16))
+    want = c_oracle.lutgemm_gemv(xn, qw.numpy(), np_of(alpha), np_of(q_bias), bits, group) + \
+        c_oracle.dec_apply(xn, L["cheat"].numpy(), np_of(L["scales"]), want_rows[:k])
     check_output(np_of(out).reshape(-1), want, "fp16", ("dec_lutgemm", K, N))
     ext.destroy_dec_config(cfg)
 

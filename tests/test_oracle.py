@@ -38,6 +38,64 @@ def test_floors_c_and_numpy_restatements_agree_bitwise(c_oracle):
             assert np.array_equal(f1.view(np.uint32), f2.view(np.uint32))
 
 
+def _round_to_format(v, p, emin):
+    """Exact rational `v` rounded to nearest, ties to even, in a binary format with `p` significand bits and minimum
+    normal exponent `emin` (subnormals included; no overflow handling: the cases below stay finite)."""
+    from fractions import Fraction
+    if v == 0:
+        return Fraction(0)
+    sign = -1 if v < 0 else 1
+    v = abs(v)
+    e = v.numerator.bit_length() - v.denominator.bit_length()        # floor(log2 v) or one above
+    if Fraction(2) ** e > v:
+        e -= 1
+    e = max(e, emin)
+    ulp = Fraction(2) ** (e - p + 1)
+    q, rem = divmod(v, ulp)
+    if rem * 2 > ulp or (rem * 2 == ulp and q % 2 == 1):
+        q += 1
+    return sign * q * ulp
+
+
+@pytest.mark.parametrize("dt,p,emin", [("fp16", 11, -14), ("bf16", 8, -126), ("fp32", 24, -126)])
+def test_floors_against_exact_rational_arithmetic(dt, p, emin, c_oracle):
+    """dec.cu:117-130 evaluated with exact fractions and one explicit round-to-nearest-even per operation (the
+    subtraction and the final addition in the activation type, the multiply and the divide in float32, the cast
+    back in the activation type).  Shares no machinery with the NumPy or the C restatement: a dropped intermediate
+    rounding, a multiply done in the 16-bit type or a divide fused into the multiply changes some of these cases."""
+    from fractions import Fraction
+    T = lambda v: _round_to_format(v, p, emin)
+    F32 = lambda v: _round_to_format(v, 24, -126)
+    rng = np.random.default_rng(20241)
+    pairs = [(1.0, 0.5), (3.0, 1.0), (0.333251953125, 0.111083984375), (6.1e-5, 3.0e-5), (60000.0, 1.5), (0.5, 1.0),
+             (1.0, 1.0), (2.0 ** -20, 2.0 ** -24), (7.0, 0.0)]
+    for _ in range(300):
+        a = float(np.exp(rng.uniform(-9, 5))); b = a * float(rng.uniform(0.02, 1.0))
+        pairs.append((a, b))
+    tdt = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}[dt]
+    differing = 0
+    for a, b in pairs:
+        a = float(torch.tensor(a).to(tdt).float()); b = float(torch.tensor(b).to(tdt).float())   # representable inputs
+        fa, fb = Fraction(a), Fraction(b)
+        want = []
+        for idx in range(32):
+            if idx < 16:
+                d = T(fb - fa)
+                step = F32(F32(d * idx) / 15)
+                want.append(T(fa + T(step)))
+            else:
+                want.append(T(F32(F32(fb * (31 - idx)) / 16)))
+        want = np.array([float(w) for w in want], dtype=np.float32)
+        got = O.bucket_floors(a, b, dt)
+        assert np.array_equal(got, want), (dt, a, b, got, want)
+        assert np.array_equal(c_oracle.bucket_floors(a, b, dt), want), (dt, a, b)
+        # the pin bites: without the cast of the step back to the activation type (one rounding of a + step instead
+        # of two) some inputs give other floors
+        lazy = np.array([float(T(fa + F32(F32(T(fb - fa) * idx) / 15))) for idx in range(16)], dtype=np.float32)
+        differing += int(not np.array_equal(lazy, want[:16]))
+    assert differing > 0 or dt == "fp32"
+
+
 def test_soft_float_conversion_matches_numpy(c_oracle):
     rng = np.random.default_rng(2)
     L = c_oracle.lib()
