@@ -716,6 +716,24 @@ def main():
     }
     result["roofline_link"] = roofline_link_leg(torch, ext, protos, args.k_chunk, args.n_tb, link_leg(torch))
     drop_configs(ctxs, cfgs)
+    # Progress against the two floors of the step: the base path against the HBM peak, the compensated step against the
+    # time its residual bytes need at the zero-copy rate measured in this run (no launch can beat either).
+    ceiling_gbs = result["roofline_link"]["measured_ceiling"]
+    link_floor_us = host_bytes / ceiling_gbs / 1e3
+    result["base_frac_of_hbm_peak"] = round(weight_bytes / (base_us - zero_us) / 1e3 / 8000.0, 4)
+    result["link_floor_us_per_token"] = round(link_floor_us * scale, 1)
+    result["frac_of_link_floor"] = round(link_floor_us / dec_us, 4)
+    result["floor_us_per_token"] = round(max(link_floor_us, weight_bytes / 8000.0 / 1e3) * scale, 1)
+    # the same step at smaller k_chunk (same n_tb): where DEC fits beside the GEMVs
+    for kc in (8, 16):
+        if kc == args.k_chunk:
+            continue
+        ctxs, cfgs = make_configs(args.n_tb, kc)
+        us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2)
+        result[f"k_chunk_{kc}_us_per_token"] = round(us * scale, 1)
+        result[f"k_chunk_{kc}_dec_slowdown_pct"] = round((us / base_us - 1) * 100, 1)
+        result[f"k_chunk_{kc}_link_floor_us_per_token"] = round(host_bytes * kc / args.k_chunk / ceiling_gbs / 1e3 * scale, 1)
+        drop_configs(ctxs, cfgs)
 
     # The same step with every layer's residual resident in HBM (a private device copy per layer: 3.3 GB, which a
     # 288 GB device holds beside the weights; the library uses a device residual in place).  Not the metric -- the

@@ -69,6 +69,7 @@ SIGNATURES = {
     "decdec_bucket_floors": [_f32, _f32, _i32, ctypes.POINTER(_f32)],
     "decdec_reference_geometry": [_u32, _u32, _u32, _u32, _i32, _u32, ctypes.POINTER(ConfigInfo)],
     "decdec_dec_launch_plan": [_u32, _u32, _u32, _u32, _u32, ctypes.POINTER(ConfigInfo)],
+    "decdec_fused_launch_form": [_i32, _i32, _u32, _u32, _u32, ctypes.POINTER(_i32)],
 }
 OTHER_SYMBOLS = {"decdec_last_error": ([], ctypes.c_char_p), "decdec_version": ([], _i32),
                  "decdec_decode_attention_workspace_bytes": ([_u32, _u32, _u32], _u64),

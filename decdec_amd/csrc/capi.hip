@@ -909,20 +909,39 @@ int decdec_sqllm_gemv(const void* input, void* output, const void* mat, const vo
 //   LUT-GEMM 5120 -> 35840:       1.4 1.9 3.1 3.4 7.2  | 11.0 11.5 12.3 15.5 17.6  beyond 1.27
 enum GemvKind { kAnyprec = 0, kLutgemm = 1, kSqllm = 2 };
 
-double dec_estimate_us(const Config* c) {
-    const double k = (double)((uint64_t)c->k_chunk * c->K / 1024u);        // selected rows per call
-    return 8.0 + k * (double)c->N * 0.5 / 56e3;
+// The outputs of a batch are merged with atomic adds by different layers' workgroups at the same time: they must
+// not overlap, not even partly (slices of one buffer are fine as long as their ranges are disjoint).
+int check_batch_outputs(uint32_t n, void* const* outputs, const uint32_t* out_features, int dtype) {
+    const size_t elem = dtype == DECDEC_FP32 ? 4 : 2;
+    for (uint32_t i = 0; i < n; ++i) {
+        DD_CHECK(outputs[i] != nullptr, "null pointer argument");
+        const uintptr_t a0 = (uintptr_t)outputs[i], a1 = a0 + (size_t)out_features[i] * elem;
+        for (uint32_t j = 0; j < i; ++j) {
+            const uintptr_t b0 = (uintptr_t)outputs[j], b1 = b0 + (size_t)out_features[j] * elem;
+            DD_CHECK(a1 <= b0 || b1 <= a0, "the outputs of layers %u and %u of a batch overlap", j, i);
+        }
+    }
+    return kOk;
 }
+
+double dec_estimate_shape_us(uint32_t K, uint32_t N, uint32_t k_chunk) {
+    const double k = (double)((uint64_t)k_chunk * K / 1024u);              // selected rows per call
+    return 8.0 + k * (double)N * 0.5 / 56e3;
+}
+double dec_estimate_us(const Config* c) { return dec_estimate_shape_us(c->K, c->N, c->k_chunk); }
 double gemv_estimate_us(GemvKind kind, double weight_bytes) {
     if (kind == kAnyprec) return 2.8 + weight_bytes / 3.7e6;
     if (kind == kSqllm) return 3.4 + weight_bytes / 4.6e6;
     return 4.2 + weight_bytes / 3.1e6;
 }
 
-bool fused_two_per_cu(const Config* c, GemvKind kind, double weight_bytes) {
+bool fused_two_per_cu_at(double dec_us, GemvKind kind, double weight_bytes) {
     if (g_opt.fused_two_per_cu >= 0) return g_opt.fused_two_per_cu != 0;
     const double flip = kind == kAnyprec ? 0.9 : (kind == kSqllm ? 1.15 : 1.3);
-    return dec_estimate_us(c) < flip * gemv_estimate_us(kind, weight_bytes);
+    return dec_us < flip * gemv_estimate_us(kind, weight_bytes);
+}
+bool fused_two_per_cu(const Config* c, GemvKind kind, double weight_bytes) {
+    return fused_two_per_cu_at(dec_estimate_us(c), kind, weight_bytes);
 }
 
 // Whether a fused 3-bit any-precision launch runs both roles in workgroups of `nw` waves (the GEMV's standalone
@@ -934,10 +953,28 @@ bool fused_two_per_cu(const Config* c, GemvKind kind, double weight_bytes) {
 // 4 / 8 / 10 / 12 / 16 against 6.6 / 6.4 / 6.4 / 6.4 / 7.1 us: the switch sits where DEC is estimated at 1.7 x the
 // GEMV (k_chunk 14 there).  With 4-wave workgroups (K <= 8192) the 1024-thread form was as fast or faster at every
 // k_chunk.
-bool fused_small(const Config* c, double gemv_bytes, uint32_t nw) {
+bool fused_small_at(double dec_us, double gemv_bytes, uint32_t nw) {
     if (nw >= 16u || g_opt.fused_small == 0) return false;
     if (g_opt.fused_small > 0) return true;
-    return nw == 8u && dec_estimate_us(c) < 1.7 * gemv_estimate_us(kAnyprec, gemv_bytes);
+    return nw == 8u && dec_us < 1.7 * gemv_estimate_us(kAnyprec, gemv_bytes);
+}
+bool fused_small(const Config* c, double gemv_bytes, uint32_t nw) { return fused_small_at(dec_estimate_us(c), gemv_bytes, nw); }
+
+int decdec_fused_launch_form(int kind, int bits, uint32_t K, uint32_t N, uint32_t k_chunk, int* form_out) {
+    DD_CHECK(form_out != nullptr, "form_out must not be null");
+    DD_CHECK(kind >= 0 && kind <= 2, "kind must be 0 (any-precision), 1 (LUT-GEMM) or 2 (SqueezeLLM)");
+    DD_CHECK(K >= 32 && K % 32 == 0 && N >= 1 && bits >= 1 && bits <= 8, "invalid shape");
+    const double dec_us = dec_estimate_shape_us(K, N, k_chunk), bytes = (double)bits * N * K / 8.0;
+    if (kind == kAnyprec && bits == 3 && g_opt.fused_small != 0) {
+        // the workgroup size the standalone 3-bit kernel would use for this shape (plan_anyprec, four rows per wave)
+        const uint32_t s_total = cdiv(K / 32u, 64u), sgroups = cdiv(s_total, 16u), S = cdiv(s_total, sgroups);
+        const uint32_t block = 64u * S * std::max(1u, 4u / S);
+        const uint32_t nw = block <= 256u ? 4u : (block <= 512u ? 8u : 16u);
+        if (fused_small_at(dec_us, bytes, nw)) { *form_out = 2; return kOk; }
+    }
+    const bool two = (kind != kAnyprec || bits == 3) && fused_two_per_cu_at(dec_us, (GemvKind)kind, bytes);
+    *form_out = two ? 1 : 0;
+    return kOk;
 }
 
 int decdec_dec_anyprec(uint64_t h, const void* input, void* output, const void* qweight, const void* lut,
@@ -993,9 +1030,7 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
     DD_CHECK(n >= 1 && n <= (uint32_t)kMaxBatch, "a batch holds 1 to %d layers, got %u", kMaxBatch, n);
     DD_CHECK(outputs && qweights && luts && out_features, "null pointer argument");
     DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
-    for (uint32_t i = 0; i < n; ++i)
-        for (uint32_t j = 0; j < i; ++j)
-            DD_CHECK(outputs[i] != outputs[j], "the layers of a batch must have distinct outputs");
+    { const int rc_out = check_batch_outputs(n, outputs, out_features, dtype); if (rc_out != kOk) return rc_out; }
     if (!g_opt.fusion || (bits != 3 && bits != 4)) {
         // no batched kernel for this case: one call per layer, same result
         for (uint32_t i = 0; i < n; ++i) {
@@ -1005,6 +1040,41 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
             if (rc != kOk) return rc;
         }
         return kOk;
+    }
+    // no DEC on any layer (no config, or k_chunk 0 everywhere): the GEMVs in their standalone workgroups, which run a
+    // batch faster than the 1024-thread workgroups of the fused kernel (gate | up at 4096 -> 14336: 13.5 against 17.3 us)
+    bool want_dec = false;
+    for (uint32_t i = 0; i < n && configs; ++i) {
+        if (!configs[i]) continue;
+        Config* c = get_config(configs[i]);
+        int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
+        if (rc != kOk) return rc;
+        want_dec = want_dec || (uint64_t)c->k_chunk * c->K / 1024u > 0;
+    }
+    if (!want_dec) {
+        GemvBatchParams<AnyprecParams> gb;
+        memset(&gb, 0, sizeof(gb));
+        gb.n = n;
+        LaunchDims gd{0, 0, 0};
+        uint32_t total = 0;
+        for (uint32_t i = 0; i < n; ++i) {
+            AnyprecPlan pl;
+            int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], false, &pl);
+            if (rc != kOk) return rc;
+            if (pl.p.tile_cs != 0u) { want_dec = true; break; }      // the tile decoder plans its own workgroups: fused form below
+            DD_CHECK(gd.block == 0 || gd.block == pl.d.block, "internal: layers of a batch planned different workgroups");
+            gb.gp[i] = pl.p;
+            gd.block = pl.d.block;
+            gd.lds = std::max(gd.lds, pl.d.lds);
+            total += pl.d.grid;
+            gb.gemv_end[i] = total;
+        }
+        if (!want_dec) {
+            for (uint32_t i = n; i < (uint32_t)kMaxBatch; ++i) gb.gemv_end[i] = total;
+            gd.grid = total;
+            DD_HIP(launch_anyprec_batch(dtype, bits, gb, gd, (hipStream_t)stream));
+            return kOk;
+        }
     }
     BatchParams<AnyprecParams> b;
     memset(&b, 0, sizeof(b));
@@ -1106,9 +1176,7 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
     DD_CHECK(n >= 1 && n <= (uint32_t)kMaxBatch, "a batch holds 1 to %d layers, got %u", kMaxBatch, n);
     DD_CHECK(outputs && out_features, "null pointer argument");
     DD_CHECK(dtype_ok(dtype), "Unsupported data type.");
-    for (uint32_t i = 0; i < n; ++i)
-        for (uint32_t j = 0; j < i; ++j)
-            DD_CHECK(outputs[i] != outputs[j], "the layers of a batch must have distinct outputs");
+    { const int rc_out = check_batch_outputs(n, outputs, out_features, dtype); if (rc_out != kOk) return rc_out; }
     if (!g_opt.fusion || !batched_kernel) {
         for (uint32_t i = 0; i < n; ++i) {
             const int rc = single(i, configs != nullptr && configs[i] != 0);
@@ -1267,9 +1335,11 @@ int decdec_rope_cache_update(const void* qkv, const void* cos_table, const void*
     return kOk;
 }
 
-static int decode_attention_common(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
-                                   void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
-                                   uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
+// Argument checks of the decode attention entry points, and the number of workgroups that share a head (1: no
+// workspace in use).  Nothing is enqueued here.
+static int decode_attention_check(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                                  void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                                  uint32_t max_seq, void* workspace, uint64_t workspace_bytes, uint32_t* nsplit_out) {
     DD_CHECK(dtype == DECDEC_FP16 || dtype == DECDEC_BF16, "Unsupported data type.");
     DD_CHECK(q && k_cache && v_cache && pos_device && out, "null pointer argument");
     DD_CHECK(n_head >= 1 && n_kv_head >= 1 && n_head % n_kv_head == 0, "n_head must be a multiple of n_kv_head");
@@ -1283,6 +1353,13 @@ static int decode_attention_common(const void* q, const void* k_cache, const voi
         DD_CHECK(((uintptr_t)workspace % 4) == 0, "workspace must be 4-byte aligned");
         nsplit = attention_splits(n_head, head_dim, workspace_bytes);
     }
+    *nsplit_out = nsplit;
+    return kOk;
+}
+
+static int decode_attention_launch(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
+                                   void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
+                                   uint32_t max_seq, void* workspace, uint32_t nsplit, void* stream) {
     AttentionParams p{q, k_cache, v_cache, (const long long*)pos_device, out, n_head, n_kv_head, head_dim, max_seq,
                       1.0f / std::sqrt((float)head_dim), nsplit, nsplit > 1 ? (float*)workspace + n_head : nullptr,
                       nullptr, nullptr, nullptr,
@@ -1295,8 +1372,12 @@ static int decode_attention_common(const void* q, const void* k_cache, const voi
 int decdec_decode_attention(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
                             void* out, int dtype, uint32_t n_head, uint32_t n_kv_head, uint32_t head_dim,
                             uint32_t max_seq, void* workspace, uint64_t workspace_bytes, void* stream) {
-    return decode_attention_common(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
-                                   workspace, workspace_bytes, stream);
+    uint32_t nsplit = 1;
+    int rc = decode_attention_check(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
+                                    workspace, workspace_bytes, &nsplit);
+    if (rc != kOk) return rc;
+    return decode_attention_launch(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
+                                   workspace, nsplit, stream);
 }
 
 int decdec_decode_attention_static(const void* q, const void* k_cache, const void* v_cache, const int64_t* pos_device,
@@ -1309,14 +1390,20 @@ int decdec_decode_attention_static(const void* q, const void* k_cache, const voi
     void* ws = nullptr;
     int rc = static_scratch(&ws);
     if (rc != kOk) return rc;
-    // The array keeps what the last call left.  Every call leaves the counters at zero; clearing the ones this call
-    // uses makes that independent of what ran before (a fill kernel, not a memset node: safe under capture).
-    if (n_head >= 1) {
+    // every argument is checked before anything is enqueued (the caller's stream may be under capture)
+    uint32_t nsplit = 1;
+    rc = decode_attention_check(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq, ws,
+                                kStaticScratchBytes, &nsplit);
+    if (rc != kOk) return rc;
+    // The array keeps what the last call left.  Every call leaves the arrival counters at zero; clearing the ones
+    // this call uses makes that independent of what ran before (a fill kernel, not a memset node: safe under
+    // capture).  They are used only when the heads are shared and merged in the kernel.
+    if (nsplit > 1 && g_opt.attention_two_step == 0) {
         hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(128), 0, (hipStream_t)stream, (uint32_t*)ws, n_head, 0u);
         DD_HIP(hipGetLastError());
     }
-    return decode_attention_common(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq,
-                                   ws, kStaticScratchBytes, stream);
+    return decode_attention_launch(q, k_cache, v_cache, pos_device, out, dtype, n_head, n_kv_head, head_dim, max_seq, ws,
+                                   nsplit, stream);
 }
 
 int decdec_rope_attention(const void* qkv, const void* cos_table, const void* sin_table, const int64_t* pos_device,

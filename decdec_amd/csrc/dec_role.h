@@ -211,7 +211,10 @@ template <int NW> struct DecTeam {
     // eight waves per SIMD (every addition to this role made that role slower); they are chosen while DEC is the
     // shorter role, and leave the rare window of more than 64 channels to the general path.
     static constexpr bool kSplit = NW >= 16;
-    static constexpr uint32_t kRank = kSplit ? kRankMax : 64u;      // candidates a team ranks (64 per ranking wave)
+    // Two ranking waves (windows of up to 128 channels) also in the 8-wave form: a window of 65 .. 128 channels is
+    // what a dense body two buckets below a sparse tail gives at small k_chunk, and the general path, run beside
+    // seven GEMV waves per SIMD, costs such a chunk 9 us (14336 -> 4096, k_chunk 6: 22.7 us instead of 13.7).
+    static constexpr uint32_t kRank = NW >= 8 ? kRankMax : 64u;     // candidates a team ranks (64 per ranking wave)
     // words of a team's area: [kAttempts][4] window counts, [4] counts at the floor inside the window,
     // [kRankMax] candidate channels, [kRankMax] candidate activations, [4] header (state, candidates, -, -)
     static constexpr int kSplitWord = 4 * kAttempts;

@@ -34,6 +34,15 @@ __global__ __launch_bounds__(1024) DD_TWO_PER_CU(TWO) void dec_anyprec_batch_ker
     }
 }
 
+// The base GEMVs of up to kMaxBatch layers on one input in one launch, in the standalone kernel's own workgroups.
+template <int DT, int BITS>
+__global__ __launch_bounds__(1024) void anyprec_batch_kernel(const GemvBatchParams<AnyprecParams> b) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    uint32_t layer, local;
+    batch_locate(b.gemv_end, blockIdx.x, layer, local);
+    anyprec_role<DT, BITS>(b.gp[layer], local, smem);
+}
+
 // The same two roles in workgroups of NW (4 or 8) waves, eight waves per SIMD: the GEMV role runs in workgroups of
 // its standalone size, and a DEC workgroup holds an eighth or a quarter of a compute unit.
 template <int DT, int NW>
@@ -132,6 +141,17 @@ hipError_t launch_dec_anyprec_batch(int dt, int bits, const BatchParams<AnyprecP
     } else {
         if (dt == kFP16) hipLaunchKernelGGL((dec_anyprec_batch_kernel<kFP16, 4, false>), grid, block, d.lds, s, b);
         else hipLaunchKernelGGL((dec_anyprec_batch_kernel<kBF16, 4, false>), grid, block, d.lds, s, b);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_anyprec_batch(int dt, int bits, const GemvBatchParams<AnyprecParams>& b, const LaunchDims& d, hipStream_t s) {
+    if (dt == kFP16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((anyprec_batch_kernel<kFP16, B>), dim3(d.grid), dim3(d.block), d.lds, s, b));
+    } else if (dt == kBF16) {
+        DD_BITS_SWITCH(bits, hipLaunchKernelGGL((anyprec_batch_kernel<kBF16, B>), dim3(d.grid), dim3(d.block), d.lds, s, b));
+    } else {
+        return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }

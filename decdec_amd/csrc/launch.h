@@ -34,6 +34,14 @@ struct BatchParams {
     DecParams dp[kMaxBatch];
     GemvParams gp[kMaxBatch];
 };
+// The base GEMVs of several layers on one input, no DEC: workgroups of the GEMV's own standalone size (a batch shares
+// its input width, so every layer plans the same workgroup), layer by layer in the grid.
+template <typename GemvParams>
+struct GemvBatchParams {
+    uint32_t n;
+    uint32_t gemv_end[kMaxBatch];
+    GemvParams gp[kMaxBatch];
+};
 // the layer a workgroup of a batch belongs to, and its index inside that layer's share of the grid
 __device__ __forceinline__ void batch_locate(const uint32_t (&end)[kMaxBatch], uint32_t id, uint32_t& layer, uint32_t& local) {
     layer = 0; local = id;
@@ -60,6 +68,9 @@ hipError_t launch_dec_anyprec(int dt, int bits, const DecParams& dp, uint32_t de
 // A batch of up to kMaxBatch any-precision layers on one input, each with or without DEC (3 or 4 bits; d.grid and
 // d.lds cover all layers; d.block is 1024).
 hipError_t launch_dec_anyprec_batch(int dt, int bits, const BatchParams<AnyprecParams>& b, const LaunchDims& d, hipStream_t s);
+// The same batch without DEC on any layer, in the standalone kernel's workgroups (d.block = the layers' common
+// workgroup size, d.grid and d.lds cover all layers; any bit width).
+hipError_t launch_anyprec_batch(int dt, int bits, const GemvBatchParams<AnyprecParams>& b, const LaunchDims& d, hipStream_t s);
 // 3-bit, both roles in workgroups of `nw` (4 or 8) waves = d.block / 64; dp carries the DEC plan for that size.
 hipError_t launch_dec_anyprec_small(int dt, uint32_t nw, const DecParams& dp, uint32_t dec_blocks,
                                     const AnyprecParams& gp, const LaunchDims& d, hipStream_t s);

@@ -52,22 +52,35 @@ typedef struct decdec_config_info {
 const char* decdec_last_error(void);
 int decdec_version(void);
 
-/* Library options: "fusion" (1 = DEC and base GEMV in one kernel launch [default], 0 = the
- * reference's two-stream fork/join, decdec.cu:621-640), "host_noncoherent" (1 = allocate the
- * pinned residual with hipHostMallocNonCoherent; default 0), "anyprec_rpw", "anyprec_tile" (3-bit LDS-transposed tile decoder for K <= 8192, waves per tile 2/4/8, 0 = off [default]), "lutgemm_ktiles",
- * "sqllm_ktiles" (launch-shape overrides, 0 = automatic), "fused_two_per_cu" (fused launches: 1 / 0 = always /
- * never the kernel instance that lets two workgroups share a compute unit, -1 = chosen per launch [default]),
- * "fused_small" (fused 3-bit any-precision launches with both roles in the GEMV's own 4- or 8-wave workgroups:
- * -1 = when those have 5 to 8 waves [default], 1 = whenever they have at most 8, 0 = never), "anyprec_rg" (row
- * groups per any-precision workgroup, 0 = automatic),
- * "attention_two_step" (decode attention with a workspace: 1 = merge in a second kernel, 0 = in the kernel [default]),
- * "attention_single_below" (... merging in the kernel: sequences of at most this many positions are scanned by one
- * workgroup per head, which is faster there; default 512, 0 = always share),
- * "dec_block_waves" (waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows),
- * "dec_max_chunk_groups" (DEC launch plans made from now on use at most this many chunk groups, i.e. atomic adds per
- * output: 1 to 4; 0 = the built-in bound of 4 [default]), "dec_force_cg" / "dec_force_sg" (DEC launch plans made from
- * now on use this many chunk groups / segment groups where the shape allows; tuning aid, 0 = planned [default]), "dec_trace" (see
- * decdec_debug_read_trace).  No counterpart in the reference. */
+/* Library options (process-wide integers).  No counterpart in the reference.
+ *
+ * Options a caller is meant to set:
+ *   "fusion"                1 = DEC and the base GEMV in one kernel launch [default]; 0 = the reference's two-stream
+ *                           fork/join (decdec.cu:621-640).
+ *   "dec_max_chunk_groups"  DEC launch plans made from now on use at most this many chunk groups, i.e. atomic adds
+ *                           (roundings of a 16-bit output in varying order) per output: 1 to 4; 1 = the reference's
+ *                           single add (dec.cu:263-276); 0 = the built-in bound of 4 [default].
+ *   "host_noncoherent"      1 = allocate the pinned residual with hipHostMallocNonCoherent; 0 [default].
+ *
+ * Experimental: launch-shape overrides and measurement aids used to tune and profile the library.  Their defaults are
+ * what the library ships with; their meaning may change with the kernels, and nothing outside a tuning session
+ * should depend on them.
+ *   "fused_two_per_cu"      fused launches: 1 / 0 = always / never the kernel instance that lets two workgroups share
+ *                           a compute unit; -1 = chosen per launch [default].
+ *   "fused_small"           fused 3-bit any-precision launches with both roles in the GEMV's own 4- or 8-wave
+ *                           workgroups: -1 = when those have 5 to 8 waves and DEC is the shorter role [default],
+ *                           1 = whenever they have at most 8 waves, 0 = never.
+ *   "dec_block_waves"       waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows.
+ *   "dec_force_cg", "dec_force_sg"   DEC launch plans made from now on use this many chunk groups / segment groups
+ *                           where the shape allows; 0 = planned [default].
+ *   "anyprec_rpw", "anyprec_rg", "lutgemm_ktiles", "sqllm_ktiles"   rows per wave / row groups per workgroup / K ranges
+ *                           of the base GEMVs; 0 = automatic [default].  (sqllm_ktiles = 1 and lutgemm_ktiles = 1 give
+ *                           every output a single atomic add from the GEMV.)
+ *   "anyprec_tile"          3-bit LDS-transposed tile decoder for K <= 8192, waves per tile 2 / 4 / 8; 0 = off [default].
+ *   "attention_two_step"    decode attention with a workspace: 1 = merge in a second kernel, 0 = in the kernel [default].
+ *   "attention_single_below"  ... merging in the kernel: sequences of at most this many positions are scanned by one
+ *                           workgroup per head; default 512, 0 = always share.
+ *   "dec_trace"             see decdec_debug_read_trace. */
 int decdec_set_option(const char* name, int value);
 int decdec_get_option(const char* name, int* value);
 
@@ -157,12 +170,14 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
 /* Several any-precision layers that read the SAME input vector, in one launch: q | k | v and gate | up of a decoder
  * layer are independent given their input, and one launch pays the launch and selection latencies once instead of once
  * per layer.  Layer i: config configs[i] (0, or a config with k_chunk 0: base GEMV only; configs may be NULL when no
- * layer has DEC), output outputs[i] (out_features[i] elements, distinct per layer, zeroed by the caller as for the
- * single-layer ops), qweights[i], luts[i].  1 to 4 layers, the same bitwidth and dtype; results are those of n
+ * layer has DEC), output outputs[i] (out_features[i] elements; the ranges of different layers must not overlap, not
+ * even partly; zeroed by the caller as for the single-layer ops), qweights[i], luts[i].  1 to 4 layers, the same bitwidth and dtype; results are those of n
  * decdec_dec_anyprec / decdec_anyprec_gemv calls.  Configs of one batch that belong to the same context write their
  * selections into the same scratch buffers at the same time: give each layer of a batch a context of its own if the
- * selection is read back.  No counterpart in the reference, which fuses such projections by concatenating their
- * weights (end-to-end/model.py wqkv, w1w3). */
+ * selection is read back.  Every layer with DEC brings the DEC workgroups of its own launch plan, each planned against
+ * its context's whole num_tb: a batch of n such layers occupies up to n x num_tb workgroups with DEC, not num_tb.
+ * No counterpart in the reference, which fuses such projections by concatenating their weights (end-to-end/model.py
+ * wqkv, w1w3). */
 int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
                              const void* const* qweights, const void* const* luts, int bitwidth, int dtype,
                              uint32_t in_features, const uint32_t* out_features, void* stream);
@@ -274,6 +289,13 @@ int decdec_reference_geometry(uint32_t num_rows, uint32_t num_cols, uint32_t num
  * group, no grid barrier). */
 int decdec_dec_launch_plan(uint32_t num_rows, uint32_t num_cols, uint32_t num_tb, uint32_t k_chunk,
                            uint32_t block_waves, decdec_config_info* info_out);
+/* Which instance of the fused DEC + GEMV kernel a single-layer call launches for a shape under the current options:
+ * 0 = 1024-thread workgroups, one per compute unit; 1 = 1024-thread workgroups, two per compute unit; 2 = both roles
+ * in the GEMV's own 4- or 8-wave workgroups (3-bit any-precision only).  kind: 0 any-precision, 1 LUT-GEMM,
+ * 2 SqueezeLLM.  Host-only; the choice rests on time estimates of the two roles, not on data.  No counterpart in
+ * the reference. */
+int decdec_fused_launch_form(int kind, int bitwidth, uint32_t in_features, uint32_t out_features, uint32_t k_chunk,
+                             int* form_out);
 
 #ifdef __cplusplus
 }

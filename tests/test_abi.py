@@ -39,7 +39,7 @@ def test_version_and_options():
         _lib.set_option("no_such_option", 1)
     # every option the header names exists, with the documented default
     header = open(os.path.join(os.path.dirname(__file__), "..", "include", "decdec_hip.h")).read()
-    block = header[header.index("/* Library options:"):header.index("int decdec_set_option")]
+    block = header[header.index("/* Library options"):header.index("int decdec_set_option")]
     named = set(re.findall(r'"([a-z0-9_]+)"', block))
     defaults = {"fusion": 1, "host_noncoherent": 0, "anyprec_rpw": 0, "anyprec_tile": 0, "lutgemm_ktiles": 0,
                 "sqllm_ktiles": 0, "attention_two_step": 0, "attention_single_below": 512, "fused_two_per_cu": -1, "fused_small": -1, "anyprec_rg": 0, "dec_block_waves": 16,
@@ -47,6 +47,9 @@ def test_version_and_options():
     assert named == set(defaults), named ^ set(defaults)
     for name, value in defaults.items():
         assert _lib.get_option(name) == value, name
+    # the options a caller is meant to touch are listed apart from the tuning aids
+    public = block[:block.index("Experimental")]
+    assert set(re.findall(r'"([a-z0-9_]+)"', public)) == {"fusion", "dec_max_chunk_groups", "host_noncoherent"}
 
 
 @pytest.mark.parametrize("dt,code", [("fp16", 1), ("bf16", 2), ("fp32", 0)])
@@ -129,6 +132,49 @@ def test_dec_launch_plan_bounds_the_atomic_adds_per_output(waves):
     # only a row list that cannot fit in LDS otherwise lifts the bound (select-all at a 70B input width)
     _lib.check(lib.decdec_dec_launch_plan(28672, 8192, 32, 1024, waves, ctypes.byref(info)))
     assert info.hip_chunk_groups > MAX_CHUNK_GROUPS and info.hip_lds_bytes <= 60 * 1024
+
+
+LLAMA3_8B_MODULES = {"qkv": (4096, 6144), "o": (4096, 4096), "gu": (4096, 28672), "d": (14336, 4096)}
+
+
+@pytest.mark.parametrize("module", sorted(LLAMA3_8B_MODULES))
+def test_fused_form_and_plan_are_monotone_in_k_chunk(module):
+    """What a fused any-precision launch looks like as k_chunk grows from 1 to 12 at the Llama-3-8B module shapes
+    (the autotuner's sweep): the kernel instance only ever moves from the forms chosen while the GEMV is the longer
+    role (both roles in the GEMV's small workgroups, then two 1024-thread workgroups per compute unit) to the one
+    chosen when DEC is (one workgroup per unit), never back; and the DEC launch plan never shrinks (workgroups,
+    segment groups).  A timing cliff at one k_chunk between two cheaper neighbours therefore cannot come from the
+    choice of form or plan: at 14336 -> 4096, k_chunk 6, it came from the selection itself (a window of 65 .. 128
+    channels, which the 8-wave form used to hand to the general path)."""
+    lib = _lib.load()
+    K, N = LLAMA3_8B_MODULES[module]
+    form = ctypes.c_int(0)
+    info = _lib.ConfigInfo()
+    order = {2: 0, 1: 1, 0: 2}                       # small workgroups -> two per unit -> one per unit
+    forms, plans = [], []
+    for k_chunk in range(1, 13):
+        _lib.check(lib.decdec_fused_launch_form(0, 3, K, N, k_chunk, ctypes.byref(form)))
+        forms.append(form.value)
+        waves = {2: 8, 1: 16, 0: 16}[form.value]
+        _lib.check(lib.decdec_dec_launch_plan(K, N, 32, k_chunk, waves, ctypes.byref(info)))
+        plans.append((form.value, info.hip_dec_blocks, info.hip_segment_groups, info.hip_chunk_groups))
+    assert all(order[a] <= order[b] for a, b in zip(forms, forms[1:])), forms
+    for (fa, ba, sa, ca), (fb, bb, sb, cb) in zip(plans, plans[1:]):
+        if fa == fb:
+            assert bb >= ba and sb >= sa and cb >= ca, plans
+    if module == "d":
+        assert forms[0] == 2 and forms[5] == 2          # the down projection starts in its 8-wave form, also at k_chunk 6
+    # the forced settings are honoured
+    for opt, val, want in (("fused_small", 0, {0, 1}), ("fused_two_per_cu", 0, {0, 2}), ("fused_two_per_cu", 1, {1, 2})):
+        _lib.set_option(opt, val)
+        try:
+            got = set()
+            for k_chunk in range(1, 13):
+                _lib.check(lib.decdec_fused_launch_form(0, 3, K, N, k_chunk, ctypes.byref(form)))
+                got.add(form.value)
+            assert got <= want, (opt, val, got)
+        finally:
+            _lib.set_option(opt, -1)
 
 
 def test_invalid_handles_and_arguments_fail_cleanly():
