@@ -68,6 +68,7 @@ struct Options {
                                 // -1 = when those have 5..8 waves (measured faster there), 1 = whenever they have <= 8, 0 = never
     int dec_force_cg = 0, dec_force_sg = 0;  // DEC launch plans: chunk groups / segment groups fixed by hand (tuning; 0 = planned)
     int dec_max_chunk_groups = 0;  // DEC launch plans: at most this many chunk groups (atomic adds per output); 0 = the built-in bound
+    int gemv_max_k_ranges = 0;     // LUT-GEMM / SqueezeLLM launch plans: at most this many K ranges (atomic adds per output); 0 = chosen for speed
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
@@ -96,6 +97,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "attention_single_below")) return &g_opt.attention_single_below;
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     if (!strcmp(name, "dec_max_chunk_groups")) return &g_opt.dec_max_chunk_groups;
+    if (!strcmp(name, "gemv_max_k_ranges")) return &g_opt.gemv_max_k_ranges;
     if (!strcmp(name, "dec_force_cg")) return &g_opt.dec_force_cg;
     if (!strcmp(name, "dec_force_sg")) return &g_opt.dec_force_sg;
     return nullptr;
@@ -474,7 +476,9 @@ int plan_lutgemm(const void* input, void* output, const void* qw, const void* al
         // workgroup slots this layer can count on: the whole device, or its share of it inside a batched launch
         const uint32_t slots = slots_avail ? slots_avail : 2u * device_cus();
         uint32_t best_cost = ~0u;
-        for (uint32_t kr = 1; kr <= 9; ++kr) {
+        // option gemv_max_k_ranges: a caller's bound on the atomic adds per output (kept while 7 tiles per wave allow it)
+        const uint32_t kr_max = g_opt.gemv_max_k_ranges >= 1 ? std::min(9u, (uint32_t)g_opt.gemv_max_k_ranges) : 9u;
+        for (uint32_t kr = 1; kr <= kr_max; ++kr) {
             const uint32_t slice = cdiv(tiles, kr * waves);
             if (slice > 7u) continue;
             const uint32_t k_tiles = cdiv(tiles, slice * waves);
@@ -515,6 +519,7 @@ int plan_sqllm(const void* input, void* output, const void* mat, const void* lut
     // 16-bit types: the pair table takes 68 KB of LDS, two workgroups fit a CU, so at most 512 workgroups run
     // at once; that many K ranges (measured best), fp32: enough for about 8 waves per SIMD
     uint32_t kt = dtype != DECDEC_FP32 ? 512u / std::min(512u, p.n_tiles) : cdiv(8192, p.n_tiles * waves);
+    if (g_opt.gemv_max_k_ranges >= 1) kt = std::min(kt, (uint32_t)g_opt.gemv_max_k_ranges);
     if (g_opt.sqllm_ktiles > 0) kt = (uint32_t)g_opt.sqllm_ktiles;
     kt = std::max(1u, std::min(std::min(kt, 8u), std::max(1u, K / (32u * waves))));
     p.kslice = cdiv(cdiv(K, kt * waves), 32) * 32;

@@ -60,6 +60,10 @@ int decdec_version(void);
  *   "dec_max_chunk_groups"  DEC launch plans made from now on use at most this many chunk groups, i.e. atomic adds
  *                           (roundings of a 16-bit output in varying order) per output: 1 to 4; 1 = the reference's
  *                           single add (dec.cu:263-276); 0 = the built-in bound of 4 [default].
+ *   "gemv_max_k_ranges"     LUT-GEMM and SqueezeLLM launch plans use at most this many K ranges, each of which adds
+ *                           to an output with one atomic add (the reference adds once per 32 or 128 channels,
+ *                           lutgemm.cu:143-148, sqllm.cu:115); 0 = as many as run fastest, up to 9 / 8 [default].
+ *                           LUT-GEMM rows longer than 3584 x the bound still get as many ranges as they need.
  *   "host_noncoherent"      1 = allocate the pinned residual with hipHostMallocNonCoherent; 0 [default].
  *
  * Experimental: launch-shape overrides and measurement aids used to tune and profile the library.  Their defaults are

@@ -43,13 +43,13 @@ def test_version_and_options():
     named = set(re.findall(r'"([a-z0-9_]+)"', block))
     defaults = {"fusion": 1, "host_noncoherent": 0, "anyprec_rpw": 0, "anyprec_tile": 0, "lutgemm_ktiles": 0,
                 "sqllm_ktiles": 0, "attention_two_step": 0, "attention_single_below": 512, "fused_two_per_cu": -1, "fused_small": -1, "anyprec_rg": 0, "dec_block_waves": 16,
-                "dec_max_chunk_groups": 0, "dec_force_cg": 0, "dec_force_sg": 0, "dec_trace": 0}
+                "dec_max_chunk_groups": 0, "gemv_max_k_ranges": 0, "dec_force_cg": 0, "dec_force_sg": 0, "dec_trace": 0}
     assert named == set(defaults), named ^ set(defaults)
     for name, value in defaults.items():
         assert _lib.get_option(name) == value, name
     # the options a caller is meant to touch are listed apart from the tuning aids
     public = block[:block.index("Experimental")]
-    assert set(re.findall(r'"([a-z0-9_]+)"', public)) == {"fusion", "dec_max_chunk_groups", "host_noncoherent"}
+    assert set(re.findall(r'"([a-z0-9_]+)"', public)) == {"fusion", "dec_max_chunk_groups", "gemv_max_k_ranges", "host_noncoherent"}
 
 
 @pytest.mark.parametrize("dt,code", [("fp16", 1), ("bf16", 2), ("fp32", 0)])

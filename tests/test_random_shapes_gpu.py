@@ -102,3 +102,38 @@ def test_base_gemvs_on_random_shapes(seed, c_oracle):
         mre, mae = rel_err(np_of(out).reshape(-1), want)
         print(f"{(seed, case, kind, K, N, bits, dt)}: max rel err {mre:.3e} (bound {TOL[dt]:.0e}), mean abs err {mae:.3e}")
         assert mre <= TOL[dt], (seed, case, kind, K, N, bits, dt, mre, mae)
+
+
+@pytest.mark.parametrize("bits,dt", [(1, "fp16"), (4, "bf16"), (3, "fp16")])
+def test_long_rows_with_bounded_k_ranges(bits, dt, c_oracle):
+    """LUT-GEMM at K = 14336, group 32: the launch plan picks seven K ranges for speed, i.e. seven roundings of a
+    16-bit output by atomic adds in varying order, and two random cases of this family once measured just over the
+    bound (1 bit fp16 1.1e-2, 4 bits bf16 8.5e-2).  With option gemv_max_k_ranges = 4 the same cases sit inside it
+    with room to spare; SqueezeLLM at the same K takes the option too.  (The default plan's figure is printed, not
+    judged.)"""
+    K, N, group = 14336, 1000, 32
+    g = torch.Generator().manual_seed(1000 * bits + len(dt))
+    x = F.make_activation(K, g, dtype=TORCH[dt])
+    words = lambda *shape: torch.randint(-2 ** 31, 2 ** 31 - 1, shape, generator=g, dtype=torch.int64).to(torch.int32)
+    qw = words(K // 32, bits, N)
+    alpha = (torch.rand(K // group, bits, N, generator=g) * 0.02).to(TORCH[dt])
+    qb = (torch.randn(K // group, N, generator=g) * 0.01).to(TORCH[dt])
+    want = c_oracle.lutgemm_gemv(np_of(x), qw.numpy(), np_of(alpha), np_of(qb), bits, group, dt)
+    mat, lut = words(K * 4 // 32, N), (torch.randn(N, 16, generator=g) * 0.05).to(TORCH[dt])
+    want_sq = c_oracle.sqllm_gemv(np_of(x), mat.numpy(), np_of(lut), 4, dt)
+    seen = {}
+    try:
+        for cap in (0, 4, 1):
+            _lib.set_option("gemv_max_k_ranges", cap)
+            out = torch.zeros(1, 1, N, dtype=TORCH[dt], device="cuda")
+            ext.lutgemm_gemv(x.cuda(), out, qw.cuda(), alpha.cuda(), qb.cuda(), bits, group)
+            out_sq = torch.zeros(1, 1, N, dtype=TORCH[dt], device="cuda")
+            ext.sqllm_gemv(x.cuda(), out_sq, mat.cuda(), lut.cuda(), 4)
+            torch.cuda.synchronize()
+            seen[cap] = (rel_err(np_of(out).reshape(-1), want)[0], rel_err(np_of(out_sq).reshape(-1), want_sq)[0])
+    finally:
+        _lib.set_option("gemv_max_k_ranges", 0)
+    print(f"K ranges by speed / at most 4 / one: LUT-GEMM {seen[0][0]:.3e} / {seen[4][0]:.3e} / {seen[1][0]:.3e}, "
+          f"SqueezeLLM {seen[0][1]:.3e} / {seen[4][1]:.3e} / {seen[1][1]:.3e} (bound {TOL[dt]:.0e})")
+    assert seen[4][0] <= 0.75 * TOL[dt] and seen[4][1] <= 0.75 * TOL[dt], seen
+    assert seen[1][1] <= 0.5 * TOL[dt], seen        # one range: a single rounding (LUT-GEMM needs at least four at this K)
