@@ -389,7 +389,8 @@ int check_dec_call(const Config* c, int dtype, uint32_t in_features, uint32_t ou
 struct AnyprecPlan { AnyprecParams p; LaunchDims d; };
 
 int plan_anyprec(const void* input, void* output, const void* qweight, const void* lut, int bits, int dtype,
-                 uint32_t K, uint32_t N, bool fused_block, AnyprecPlan* pl, uint32_t rpw_cap = 8) {
+                 uint32_t K, uint32_t N, bool fused_block, AnyprecPlan* pl, uint32_t rpw_cap = 8,
+                 uint64_t rows_in_launch = 0) {
     DD_CHECK(bits >= 3 && bits <= 8, "Bitwidth must be between 3 and 8.");
     if (dtype == DECDEC_FP32)
         return fail(kUnsupported, "Any-Precision GEMV does not support float data type. Please use half or bfloat16.");
@@ -410,7 +411,9 @@ int plan_anyprec(const void* input, void* output, const void* qweight, const voi
     // Rows per wave: every wave requests all its rows at once, so more rows per wave mean more bytes
     // in flight per resident wave (large matrices), fewer rows mean more waves to share the decode
     // work (small matrices, where one wave per SIMD would issue at a quarter of the VALU rate).
-    const uint64_t row_slices = (uint64_t)N * p.S * p.sgroups;
+    // (a layer of a batched launch is planned by the rows of the whole launch: two 14336-row layers planned alone get
+    // four rows per wave and 3584 workgroups between them, whose dispatch alone outlasts the 1792 of eight rows per wave)
+    const uint64_t row_slices = std::max<uint64_t>(N, rows_in_launch) * p.S * p.sgroups;
     uint32_t rpw = row_slices >= 32768 ? 8u : (row_slices >= 8192 ? 4u : 2u);
     if (row_slices >= 16384 && p.S * p.sgroups >= 4) rpw = 8u;     // long rows (K >= 8192): measured 9.0 against 10.1 us at 14336 -> 4096
     if (g_opt.anyprec_rpw == 2 || g_opt.anyprec_rpw == 4 || g_opt.anyprec_rpw == 8) rpw = (uint32_t)g_opt.anyprec_rpw;
@@ -1062,9 +1065,11 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
         gb.n = n;
         LaunchDims gd{0, 0, 0};
         uint32_t total = 0;
+        uint64_t rows = 0;
+        for (uint32_t i = 0; i < n; ++i) rows += out_features[i];
         for (uint32_t i = 0; i < n; ++i) {
             AnyprecPlan pl;
-            int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], false, &pl);
+            int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], false, &pl, 8, rows);
             if (rc != kOk) return rc;
             if (pl.p.tile_cs != 0u) { want_dec = true; break; }      // the tile decoder plans its own workgroups: fused form below
             DD_CHECK(gd.block == 0 || gd.block == pl.d.block, "internal: layers of a batch planned different workgroups");
@@ -1088,6 +1093,8 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
     uint32_t dec_total = 0, gemv_total = 0;
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
+    uint64_t batch_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) batch_rows += out_features[i];
     for (uint32_t i = 0; i < n; ++i) {
         Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
         bool have_dec = false;
@@ -1098,7 +1105,7 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
             b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
         }
         AnyprecPlan pl;
-        int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], true, &pl);
+        int rc = plan_anyprec(input, outputs[i], qweights[i], luts[i], bits, dtype, K, out_features[i], true, &pl, 8, batch_rows);
         if (rc != kOk) return rc;
         b.gp[i] = pl.p;
         d.lds = std::max(d.lds, pl.d.lds);
@@ -1196,6 +1203,8 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
     uint32_t dec_total = 0, gemv_total = 0;
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
+    uint64_t batch_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) batch_rows += out_features[i];
     for (uint32_t i = 0; i < n; ++i) {
         Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
         bool have_dec = false;
