@@ -388,6 +388,29 @@ def test_batched_launch_at_the_benchmark_shapes(Ns, two_per_cu, c_oracle):
         _lib.set_option("fused_two_per_cu", -1)
 
 
+@pytest.mark.parametrize("K,Ns,bits", [(4096, (14336, 14336), 3), (4096, (4096, 1024, 1024), 3), (4096, (14336, 40, 1000), 3),
+                                       (2080, (3000, 17, 7000, 64), 3), (4096, (6000, 24, 1000), 4)],
+                         ids=["gate_up", "q_k_v", "ragged", "ragged_k_tail", "ragged_4bit"])
+def test_base_only_batch_planned_by_its_total_rows(K, Ns, bits, c_oracle):
+    """A batch without DEC runs the layers' GEMVs in one launch of the standalone kernel's workgroups, every layer with
+    the rows per wave that the rows of the whole launch call for: a 40-row layer beside a 14336-row one gets eight rows
+    per wave and row tails in every workgroup.  Every output against the oracle."""
+    g = torch.Generator().manual_seed(sum(Ns) + K + bits)
+    x = F.make_activation(K, g)
+    xn = np_of(x)
+    qws, luts, wants = [], [], []
+    for N in Ns:
+        qweight = torch.randint(-2 ** 31, 2 ** 31 - 1, (bits, N, K // 32), generator=g, dtype=torch.int64).to(torch.int32).contiguous()
+        lut = (torch.randn(N, 2 ** bits, generator=g) * 0.02).sort(dim=1).values.half().contiguous()
+        wants.append(c_oracle.anyprec_gemv(xn, qweight.numpy(), np_of(lut), bits))
+        qws.append(qweight.cuda()); luts.append(lut.cuda())
+    outs = [torch.zeros(1, 1, N, dtype=torch.float16, device="cuda") for N in Ns]
+    ext.dec_anyprec_batch(None, x.cuda(), outs, qws, luts, bits)
+    torch.cuda.synchronize()
+    for li, want in enumerate(wants):
+        check_output(np_of(outs[li]).reshape(-1), want, "fp16", (K, Ns, bits, li))
+
+
 @pytest.mark.parametrize("K,N", [(28672, 8192), (8192, 28672)])
 def test_anyprec_at_llama3_70b_gate_and_down(K, N, c_oracle):
     """Any-precision 3-bit at the two large 70B linears (28672 -> 8192 is the 14-slice, 896-thread launch form):
