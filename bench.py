@@ -97,10 +97,26 @@ def capture(torch, fn):
     return graph
 
 
-def time_graph(torch, graph, steps, warmup):
+SETTLE_MS = 40.0    # the shader clock takes some tens of milliseconds of load to settle; a shorter run times the ramp
+
+
+def settle(torch, graph, ms=SETTLE_MS):
+    """Replays `graph` (on the current stream) until `ms` of wall time have passed."""
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(4):
+            graph.replay()
+        torch.cuda.synchronize()
+
+
+def time_graph(torch, graph, steps, warmup, settle_ms=0.0):
+    """Wall-clock microseconds per replay over exactly `steps` replays after `warmup` untimed ones; `settle_ms` > 0
+    (the secondary legs) keeps warming until that much time has passed."""
     for _ in range(warmup):
         graph.replay()
     torch.cuda.synchronize()
+    if settle_ms > 0:
+        settle(torch, graph, settle_ms)
     t0 = time.perf_counter()
     for _ in range(steps):
         graph.replay()
@@ -123,9 +139,12 @@ def measured_traffic():
     return None
 
 
-def event_time_us(torch, stream, graph, reps):
-    """Average microseconds per replay of `graph`, HIP events on the stream the graph is launched on."""
+def event_time_us(torch, stream, graph, reps, settle_ms=SETTLE_MS):
+    """Average microseconds per replay of `graph`, HIP events on the stream the graph is launched on, after
+    `settle_ms` of untimed replays."""
     with torch.cuda.stream(stream):
+        if settle_ms > 0:
+            settle(torch, graph, settle_ms)
         a = torch.cuda.Event(enable_timing=True)
         b = torch.cuda.Event(enable_timing=True)
         a.record(stream)
@@ -349,18 +368,7 @@ def kernels_leg(torch, ext, F):
         with torch.cuda.graph(gr, stream=st):
             for _ in range(reps):
                 fn()
-        for _ in range(3):
-            gr.replay()
-        torch.cuda.synchronize()
-        a = torch.cuda.Event(enable_timing=True)
-        b = torch.cuda.Event(enable_timing=True)
-        with torch.cuda.stream(st):
-            a.record(st)
-            for _ in range(iters):
-                gr.replay()
-            b.record(st)
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / iters / reps * 1e3
+        return event_time_us(torch, st, gr, iters) / reps
 
     def dec_cfg(K, N, kc, ntb):
         rows = torch.zeros(K, dtype=torch.int32, device=dev)
@@ -561,7 +569,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=32, help="decoder layers per token (32 = Llama-3-8B)")
     ap.add_argument("--k-chunk", type=int, default=32)
     ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
@@ -681,14 +689,16 @@ def main():
     for name, launch, batch in (("base", base_launch, base_batch), ("dec", dec_launch, dec_batch)):
         for mode in ("batched", "serial", "branches"):
             g = capture(torch, lambda: run_step(launch, mode, batch))
-            times[(name, mode)] = time_graph(torch, g, args.steps, args.warmup)
+            # the headline leg does exactly --warmup untimed steps; the others also warm until the clock has settled
+            times[(name, mode)] = time_graph(torch, g, args.steps, args.warmup,
+                                             0.0 if (name, mode) == ("dec", "batched") else SETTLE_MS)
             del g
     base_us, dec_us = times[("base", "batched")], times[("dec", "batched")]
     scale = 32.0 / args.layers
 
     # clearing the outputs is part of the layer contract (the kernels accumulate), so the arena fill stays
     # inside the timed region; its share is reported
-    zero_us = time_graph(torch, capture(torch, lambda: arena.zero_()), args.steps, args.warmup)
+    zero_us = time_graph(torch, capture(torch, lambda: arena.zero_()), args.steps, args.warmup, SETTLE_MS)
 
     weight_bytes = sum(anyprec_bytes(l["K"], l["N"]) for l in layers)
     host_bytes = sum(args.k_chunk * l["K"] // 1024 * l["N"] // 2 for l in layers)
@@ -729,7 +739,7 @@ def main():
         if kc == args.k_chunk:
             continue
         ctxs, cfgs = make_configs(args.n_tb, kc)
-        us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2)
+        us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2, SETTLE_MS)
         result[f"k_chunk_{kc}_us_per_token"] = round(us * scale, 1)
         result[f"k_chunk_{kc}_dec_slowdown_pct"] = round((us / base_us - 1) * 100, 1)
         result[f"k_chunk_{kc}_link_floor_us_per_token"] = round(host_bytes * kc / args.k_chunk / ceiling_gbs / 1e3 * scale, 1)
@@ -750,7 +760,7 @@ def main():
         os.close(null_fd)
         os.close(err_fd)
     cfgs = dev_cfgs
-    dev_us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), args.steps, args.warmup)
+    dev_us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), args.steps, args.warmup, SETTLE_MS)
     result["residual_in_hbm_us_per_token"] = round(dev_us * scale, 2)
     result["residual_in_hbm_dec_slowdown_pct"] = round((dev_us / base_us - 1) * 100, 2)
     drop_configs(dev_ctxs, dev_cfgs)
@@ -760,7 +770,7 @@ def main():
         for n_tb in (8, 16, 32, 64):
             for k_chunk in (8, 16, 32, 64):
                 ctxs, cfgs = make_configs(n_tb, k_chunk)
-                us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2)
+                us = time_graph(torch, capture(torch, lambda: run_step(dec_launch, "batched", dec_batch)), max(5, args.steps // 2), 2, SETTLE_MS)
                 sweep.append({"n_tb": n_tb, "k_chunk": k_chunk, "us_per_token": round(us * scale, 1),
                               "slowdown_pct": round((us / base_us - 1) * 100, 1)})
                 drop_configs(ctxs, cfgs)
