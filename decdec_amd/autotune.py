@@ -20,6 +20,7 @@ the parameters:
 from __future__ import annotations
 
 import argparse
+import time
 import json
 import sys
 
@@ -117,7 +118,7 @@ def tune(results: dict, target_slowdown: float, matrix_dims: dict) -> dict:
 # measurement (GPU)
 # ----------------------------------------------------------------------------------------------------
 def measure(matrix_dims: dict, algo: str, bitwidth: int, n_tb_values, k_chunk_values, group_size: int = 128,
-            reps: int = 10, iters: int = 10, log=None) -> dict:
+            reps: int = 10, iters: int = 10, log=None, settle_ms: float = 20.0) -> dict:
     """Times base GEMV and fused DEC + GEMV of every module on synthetic data (fp16)."""
     import torch
     from . import ext, formats as F
@@ -135,8 +136,12 @@ def measure(matrix_dims: dict, algo: str, bitwidth: int, n_tb_values, k_chunk_va
         with torch.cuda.graph(gr, stream=st):
             for _ in range(reps):
                 fn()
-        gr.replay()
-        torch.cuda.synchronize()
+        # the shader clock takes some tens of milliseconds of load to settle after an idle period (the set-up between two
+        # points is one): replay untimed first, or neighbouring points are timed at different clocks
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < settle_ms:
+            gr.replay()
+            torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         with torch.cuda.stream(st):
             a.record(st)
