@@ -341,7 +341,7 @@ int setup_config(Config* c, uint32_t k_chunk) {
 const DecPlan& dec_plan(const Config* c, uint32_t nw) { return c->plans[nw <= 4 ? 0 : (nw <= 8 ? 1 : 2)]; }
 
 int fill_dec_params(const Config* c, const void* input, void* output, bool fused_select, DecParams* p,
-                    uint32_t nw = kDecWaves) {
+                    uint32_t nw = kDecWaves, const DecPlan* plan_override = nullptr) {
     const uint64_t k = (uint64_t)c->k_chunk * c->K / 1024;       // reference decdec.cu:50
     if (k == 0) return 1;                                        // reference decdec.cu:52-54
     memset(p, 0, sizeof(*p));
@@ -358,7 +358,7 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
     }
     p->K = c->K; p->N = c->N; p->M = c->M;
     p->num_chunks = cdiv(c->K, 1024); p->k_chunk = c->k_chunk; p->k_total = (uint32_t)k;
-    const DecPlan& plan = dec_plan(c, nw);
+    const DecPlan& plan = plan_override ? *plan_override : dec_plan(c, nw);
     p->cg = plan.cg; p->sg = plan.sg; p->nseg = plan.nseg;
     p->segs_per_block = plan.segs_per_block; p->slots_per_block = plan.slots;
     p->fused_select = fused_select ? 1u : 0u;
@@ -368,6 +368,16 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
         p->trace = g_trace_dev;
     }
     return 0;
+}
+
+// DEC plan of one layer of a batched launch (1024-thread workgroups).  The layers of a batch share their contexts'
+// workgroup budget by output width, with a floor of eight workgroups per layer.  Measured on the Llama-3-8B linear set at
+// k_chunk 32, num_tb 32: gate | up planned with the whole budget each (2 x 28 DEC workgroups) 2951-2982 us per token,
+// with 2 x 16 to 2 x 24 workgroups 2896-2904, with 2 x 12 2991; a layer launched alone is best with its full budget.
+int plan_dec_in_batch(const Config* c, uint64_t dec_rows_in_batch, DecPlan* pl) {
+    const uint64_t num_tb = std::max(1u, c->ctx->num_tb);
+    const uint32_t share = (uint32_t)std::min<uint64_t>(num_tb, std::max<uint64_t>(8, num_tb * c->N / std::max<uint64_t>(1, dec_rows_in_batch)));
+    return plan_dec(c->K, c->M, c->k_chunk, share, kDecWaves, pl);
 }
 
 int check_dec_call(const Config* c, int dtype, uint32_t in_features, uint32_t out_features,
@@ -1093,15 +1103,23 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
     uint32_t dec_total = 0, gemv_total = 0;
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
-    uint64_t batch_rows = 0;
-    for (uint32_t i = 0; i < n; ++i) batch_rows += out_features[i];
+    uint64_t batch_rows = 0, dec_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        batch_rows += out_features[i];
+        if (configs && configs[i]) {
+            const Config* c = get_config(configs[i]);
+            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) dec_rows += out_features[i];
+        }
+    }
     for (uint32_t i = 0; i < n; ++i) {
         Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
         bool have_dec = false;
+        DecPlan dplan{};
         if (configs && configs[i]) {
             int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
             if (rc != kOk) return rc;
-            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i]) == 0;
+            DD_CHECK(plan_dec_in_batch(c, dec_rows, &dplan) == 0, "internal: no DEC plan for a layer of the batch");
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan) == 0;
             b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
         }
         AnyprecPlan pl;
@@ -1110,8 +1128,8 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
         b.gp[i] = pl.p;
         d.lds = std::max(d.lds, pl.d.lds);
         if (have_dec) {
-            dec_total += c->plans[2].cg * c->plans[2].sg;
-            d.lds = std::max(d.lds, c->plans[2].lds);
+            dec_total += dplan.cg * dplan.sg;
+            d.lds = std::max(d.lds, dplan.lds);
             dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
             any_dec = true;
         }
@@ -1203,15 +1221,22 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
     uint32_t dec_total = 0, gemv_total = 0;
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
-    uint64_t batch_rows = 0;
-    for (uint32_t i = 0; i < n; ++i) batch_rows += out_features[i];
+    uint64_t dec_rows = 0;
+    for (uint32_t i = 0; i < n; ++i) {
+        if (configs && configs[i]) {
+            const Config* c = get_config(configs[i]);
+            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) dec_rows += out_features[i];
+        }
+    }
     for (uint32_t i = 0; i < n; ++i) {
         Config* c = (configs && configs[i]) ? get_config(configs[i]) : nullptr;
         bool have_dec = false;
+        DecPlan dplan{};
         if (configs && configs[i]) {
             int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
             if (rc != kOk) return rc;
-            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i]) == 0;
+            DD_CHECK(plan_dec_in_batch(c, dec_rows, &dplan) == 0, "internal: no DEC plan for a layer of the batch");
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan) == 0;
             b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
         }
         LaunchDims ld{0, 0, 0};
@@ -1220,8 +1245,8 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
         DD_CHECK(ld.block == 1024u, "internal: batched layers need 1024-thread workgroups");
         d.lds = std::max(d.lds, ld.lds);
         if (have_dec) {
-            dec_total += c->plans[2].cg * c->plans[2].sg;
-            d.lds = std::max(d.lds, c->plans[2].lds);
+            dec_total += dplan.cg * dplan.sg;
+            d.lds = std::max(d.lds, dplan.lds);
             dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
             any_dec = true;
         }
