@@ -371,12 +371,14 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
 }
 
 // DEC plan of one layer of a batched launch (1024-thread workgroups).  The layers of a batch share their contexts'
-// workgroup budget by output width, with a floor of eight workgroups per layer.  Measured on the Llama-3-8B linear set at
+// workgroup budget by output width, with a floor of min(num_tb, 16) workgroups per layer.  Measured on the Llama-3-8B linear set at
 // k_chunk 32, num_tb 32: gate | up planned with the whole budget each (2 x 28 DEC workgroups) 2951-2982 us per token,
-// with 2 x 16 to 2 x 24 workgroups 2896-2904, with 2 x 12 2991; a layer launched alone is best with its full budget.
+// with 2 x 16 to 2 x 24 workgroups 2896-2904, with 2 x 12 2948-2991, with 2 x 8 2974; a layer launched alone is best with
+// its full budget.
+// Hence also the bound of 48 on what a batch shares out.
 int plan_dec_in_batch(const Config* c, uint64_t dec_rows_in_batch, DecPlan* pl) {
-    const uint64_t num_tb = std::max(1u, c->ctx->num_tb);
-    const uint32_t share = (uint32_t)std::min<uint64_t>(num_tb, std::max<uint64_t>(8, num_tb * c->N / std::max<uint64_t>(1, dec_rows_in_batch)));
+    const uint64_t num_tb = std::min(48u, std::max(1u, c->ctx->num_tb)), floor_tb = std::min<uint64_t>(num_tb, 16);
+    const uint32_t share = (uint32_t)std::min<uint64_t>(num_tb, std::max<uint64_t>(floor_tb, num_tb * c->N / std::max<uint64_t>(1, dec_rows_in_batch)));
     return plan_dec(c->K, c->M, c->k_chunk, share, kDecWaves, pl);
 }
 

@@ -179,8 +179,9 @@ int decdec_dummy_sqllm(const void* input, void* output, const void* qweight, con
  * decdec_dec_anyprec / decdec_anyprec_gemv calls.  Configs of one batch that belong to the same context write their
  * selections into the same scratch buffers at the same time: give each layer of a batch a context of its own if the
  * selection is read back.  The layers with DEC share the workgroup budget: layer i is planned against its context's
- * num_tb times its share of the batch's DEC output features, but against at least 8 workgroups, so a batch occupies
- * about num_tb workgroups with DEC (at most 8 per layer more), not n x num_tb.
+ * num_tb (48 if num_tb is larger) times its share of the batch's DEC output features, but against at least
+ * min(num_tb, 16) workgroups: a batch occupies about num_tb workgroups with DEC when num_tb is 32 or more, and up to
+ * n x num_tb when num_tb is 16 or less.
  * No counterpart in the reference, which fuses such projections by concatenating their weights (end-to-end/model.py
  * wqkv, w1w3). */
 int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* input, void* const* outputs,
