@@ -295,8 +295,11 @@ int plan_dec(uint32_t K, uint32_t M, uint32_t k_chunk, uint32_t budget, uint32_t
                 // pieces of one row are contiguous in host memory.  Measured, DEC alone at k_chunk 32 with the same
                 // number of batches: 4096 x 4096 15.3 us with 1 chunk group x 8 segment groups, 12.3 us with 4 x 2 or
                 // 4 x 8; 14336 x 4096 41.6 / 32.0 / 26.3 us with 1 / 2 / 4 chunk groups; 28672 x 8192 108 / 88 / 79 us.
+                // ... and, below sixteen workgroups, to more segment groups: measured on the Llama-3-8B token at k_chunk 8,
+                // 1540 us with 4 / 8 / 8 workgroups for the 4096-, 14336-output and down-projection launches, 1505 us with 16
+                // each (shorter merges, fewer rows per wave behind one round trip); with the residual in HBM 1539 -> 1524.
                 const uint64_t cost = batches * 1000 + (uint64_t)cdiv(cpb, teams) * 600 + (uint64_t)(64u - std::min(cg, 64u)) * 10 +
-                                      (cg * sg > budget ? 500000ull : 0);
+                                      (uint64_t)(16u - std::min(cg * sg, 16u)) * 20 + (cg * sg > budget ? 500000ull : 0);
                 if (cost < best_cost) { best_cost = cost; best_cg = cg; best_sg = sg; best_lds = lds; }
             }
         }
