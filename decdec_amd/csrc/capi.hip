@@ -947,11 +947,16 @@ int check_batch_outputs(uint32_t n, void* const* outputs, const uint32_t* out_fe
     return kOk;
 }
 
-double dec_estimate_shape_us(uint32_t K, uint32_t N, uint32_t k_chunk) {
+// Bytes per microsecond at which a DEC role reads its residual rows: the host link's measured ceiling for a residual in
+// pinned host memory; for a residual that already lives in device memory the rows cost next to nothing beside the
+// role's latency floor (measured: 8.5 us at 4096 -> 4096 and 15.7 us at 14336 -> 4096, k_chunk 32, against 11.8 and 24.5).
+constexpr double kHostLinkBytesPerUs = 56e3, kDeviceResidualBytesPerUs = 1e6;
+double dec_estimate_shape_us(uint32_t K, uint32_t N, uint32_t k_chunk, double bytes_per_us = kHostLinkBytesPerUs) {
     const double k = (double)((uint64_t)k_chunk * K / 1024u);              // selected rows per call
-    return 8.0 + k * (double)N * 0.5 / 56e3;
+    return 8.0 + k * (double)N * 0.5 / bytes_per_us;
 }
-double dec_estimate_us(const Config* c) { return dec_estimate_shape_us(c->K, c->N, c->k_chunk); }
+double dec_residual_rate(const Config* c) { return c->residual_host ? kHostLinkBytesPerUs : kDeviceResidualBytesPerUs; }
+double dec_estimate_us(const Config* c) { return dec_estimate_shape_us(c->K, c->N, c->k_chunk, dec_residual_rate(c)); }
 double gemv_estimate_us(GemvKind kind, double weight_bytes) {
     if (kind == kAnyprec) return 2.8 + weight_bytes / 3.7e6;
     if (kind == kSqllm) return 3.4 + weight_bytes / 4.6e6;
@@ -1135,7 +1140,7 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
         if (have_dec) {
             dec_total += dplan.cg * dplan.sg;
             d.lds = std::max(d.lds, dplan.lds);
-            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
+            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_residual_rate(c);
             any_dec = true;
         }
         gemv_total += pl.d.grid;
@@ -1252,7 +1257,7 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
         if (have_dec) {
             dec_total += dplan.cg * dplan.sg;
             d.lds = std::max(d.lds, dplan.lds);
-            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / 56e3;
+            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_residual_rate(c);
             any_dec = true;
         }
         gemv_total += ld.grid;
