@@ -69,6 +69,7 @@ struct Options {
     int dec_force_cg = 0, dec_force_sg = 0;  // DEC launch plans: chunk groups / segment groups fixed by hand (tuning; 0 = planned)
     int dec_max_chunk_groups = 0;  // DEC launch plans: at most this many chunk groups (atomic adds per output); 0 = the built-in bound
     int gemv_max_k_ranges = 0;     // LUT-GEMM / SqueezeLLM launch plans: at most this many K ranges (atomic adds per output); 0 = chosen for speed
+    int dec_rows_in_flight = 0;    // residual rows a DEC wave requests at a time: 2, 4 or 8; 0 = chosen per launch
     int anyprec_tile = 0;     // 3-bit tile decoder: waves per tile (2, 4, 8); 0 = off (default: the row-slice kernel is faster at decode shapes)
 } g_opt;
 
@@ -98,6 +99,7 @@ int* option_slot(const char* name) {
     if (!strcmp(name, "dec_block_waves")) return &g_opt.dec_block_waves;
     if (!strcmp(name, "dec_max_chunk_groups")) return &g_opt.dec_max_chunk_groups;
     if (!strcmp(name, "gemv_max_k_ranges")) return &g_opt.gemv_max_k_ranges;
+    if (!strcmp(name, "dec_rows_in_flight")) return &g_opt.dec_rows_in_flight;
     if (!strcmp(name, "dec_force_cg")) return &g_opt.dec_force_cg;
     if (!strcmp(name, "dec_force_sg")) return &g_opt.dec_force_sg;
     return nullptr;
@@ -343,8 +345,31 @@ int setup_config(Config* c, uint32_t k_chunk) {
 // Fill the kernel parameters of one DEC call.  Returns 1 when there is nothing to do (k == 0).
 const DecPlan& dec_plan(const Config* c, uint32_t nw) { return c->plans[nw <= 4 ? 0 : (nw <= 8 ? 1 : 2)]; }
 
+// Bytes per microsecond at which a DEC role reads its residual rows: the host link's measured ceiling for a residual in
+// pinned host memory; for a residual that already lives in device memory the rows cost next to nothing beside the
+// role's latency floor (measured: 8.5 us at 4096 -> 4096 and 15.7 us at 14336 -> 4096, k_chunk 32, against 11.8 and 24.5).
+constexpr double kHostLinkBytesPerUs = 56e3, kDeviceResidualBytesPerUs = 1e6;
+double dec_residual_rate(const Config* c) { return c->residual_host ? kHostLinkBytesPerUs : kDeviceResidualBytesPerUs; }
+
+// Residual rows a wave requests per round (dec_role.h, dec_fetch_rows): the fewest of 2, 4, 8 with which the wave's rows
+// take no more rounds than fit into the time the launch's rows occupy the link anyway (a round trip under light load is
+// about 1.5 us).  Few rows per round keep the number of requests in flight near what the link serves per round trip;
+// measured on the Llama-3-8B token with one value for every launch, k_chunk 4 / 8 / 16 / 32 / 64: 1336 / 1496 / 1882 /
+// 2808 / 4767 us with two, 1367 / 1459 / 1917 / 2912 / 4909 with four, 1400 / 1520 / 1935 / 2903 / 4866 with eight
+// (at k_chunk 8 the down projection has eight rows per wave behind 4 us of link time and wants four per round; with the
+// residual in HBM, k_chunk 64: 1874 / 1677 / 1642).
+uint32_t dec_rows_per_round(const DecPlan& plan, uint32_t nw, double launch_link_us) {
+    if (g_opt.dec_rows_in_flight > 0) return (uint32_t)g_opt.dec_rows_in_flight;
+    const uint32_t sb = std::max(1u, std::min(plan.segs_per_block, nw)), waves_per_segment = std::max(1u, nw / sb);
+    const uint32_t rows_per_wave = cdiv(plan.slots, waves_per_segment);
+    const uint32_t rounds = (uint32_t)std::max(1.0, launch_link_us / 1.5);
+    uint32_t u = 2;
+    while (u < 8u && cdiv(rows_per_wave, u) > rounds) u *= 2u;
+    return u;
+}
+
 int fill_dec_params(const Config* c, const void* input, void* output, bool fused_select, DecParams* p,
-                    uint32_t nw = kDecWaves, const DecPlan* plan_override = nullptr) {
+                    uint32_t nw = kDecWaves, const DecPlan* plan_override = nullptr, double launch_link_us = 0.0) {
     const uint64_t k = (uint64_t)c->k_chunk * c->K / 1024;       // reference decdec.cu:50
     if (k == 0) return 1;                                        // reference decdec.cu:52-54
     memset(p, 0, sizeof(*p));
@@ -365,6 +390,8 @@ int fill_dec_params(const Config* c, const void* input, void* output, bool fused
     p->cg = plan.cg; p->sg = plan.sg; p->nseg = plan.nseg;
     p->segs_per_block = plan.segs_per_block; p->slots_per_block = plan.slots;
     p->fused_select = fused_select ? 1u : 0u;
+    const double own_link_us = (double)k * (double)c->N * 0.5 / dec_residual_rate(c);
+    p->rows_in_flight = dec_rows_per_round(plan, nw, std::max(own_link_us, launch_link_us));
     if (g_opt.dec_trace && p->cg * p->sg <= (uint32_t)kTraceBlocks) {
         if (!g_trace_dev && hipMalloc(&g_trace_dev, sizeof(unsigned long long) * 8 * kTraceBlocks) != hipSuccess)
             g_trace_dev = nullptr;
@@ -947,15 +974,10 @@ int check_batch_outputs(uint32_t n, void* const* outputs, const uint32_t* out_fe
     return kOk;
 }
 
-// Bytes per microsecond at which a DEC role reads its residual rows: the host link's measured ceiling for a residual in
-// pinned host memory; for a residual that already lives in device memory the rows cost next to nothing beside the
-// role's latency floor (measured: 8.5 us at 4096 -> 4096 and 15.7 us at 14336 -> 4096, k_chunk 32, against 11.8 and 24.5).
-constexpr double kHostLinkBytesPerUs = 56e3, kDeviceResidualBytesPerUs = 1e6;
 double dec_estimate_shape_us(uint32_t K, uint32_t N, uint32_t k_chunk, double bytes_per_us = kHostLinkBytesPerUs) {
     const double k = (double)((uint64_t)k_chunk * K / 1024u);              // selected rows per call
     return 8.0 + k * (double)N * 0.5 / bytes_per_us;
 }
-double dec_residual_rate(const Config* c) { return c->residual_host ? kHostLinkBytesPerUs : kDeviceResidualBytesPerUs; }
 double dec_estimate_us(const Config* c) { return dec_estimate_shape_us(c->K, c->N, c->k_chunk, dec_residual_rate(c)); }
 double gemv_estimate_us(GemvKind kind, double weight_bytes) {
     if (kind == kAnyprec) return 2.8 + weight_bytes / 3.7e6;
@@ -1114,11 +1136,15 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
     uint64_t batch_rows = 0, dec_rows = 0;
+    double batch_link_us = 0.0;
     for (uint32_t i = 0; i < n; ++i) {
         batch_rows += out_features[i];
         if (configs && configs[i]) {
             const Config* c = get_config(configs[i]);
-            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) dec_rows += out_features[i];
+            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) {
+                dec_rows += out_features[i];
+                batch_link_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_residual_rate(c);
+            }
         }
     }
     for (uint32_t i = 0; i < n; ++i) {
@@ -1129,7 +1155,7 @@ int decdec_dec_anyprec_batch(uint32_t n, const uint64_t* configs, const void* in
             int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
             if (rc != kOk) return rc;
             DD_CHECK(plan_dec_in_batch(c, dec_rows, &dplan) == 0, "internal: no DEC plan for a layer of the batch");
-            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan) == 0;
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan, batch_link_us) == 0;
             b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
         }
         AnyprecPlan pl;
@@ -1232,10 +1258,14 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
     double dec_us = 0.0, weight_bytes = 0.0;
     bool any_dec = false;
     uint64_t dec_rows = 0;
+    double batch_link_us = 0.0;
     for (uint32_t i = 0; i < n; ++i) {
         if (configs && configs[i]) {
             const Config* c = get_config(configs[i]);
-            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) dec_rows += out_features[i];
+            if (c && (uint64_t)c->k_chunk * c->K / 1024u > 0) {
+                dec_rows += out_features[i];
+                batch_link_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_residual_rate(c);
+            }
         }
     }
     for (uint32_t i = 0; i < n; ++i) {
@@ -1246,7 +1276,7 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
             int rc = check_dec_call(c, dtype, K, out_features[i], input, outputs[i]);
             if (rc != kOk) return rc;
             DD_CHECK(plan_dec_in_batch(c, dec_rows, &dplan) == 0, "internal: no DEC plan for a layer of the batch");
-            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan) == 0;
+            have_dec = fill_dec_params(c, input, outputs[i], true, &b.dp[i], kDecWaves, &dplan, batch_link_us) == 0;
             b.dp[i].trace = nullptr;                      // the phase stamps are indexed by workgroup of a single-layer launch
         }
         LaunchDims ld{0, 0, 0};

@@ -8,8 +8,9 @@
 // (segment group).  It selects the channels of its own chunks itself -- selection needs only the
 // activation vector, so no grid-wide barrier and no second launch -- and then fetches the selected
 // residual rows restricted to its column segments.  A segment is 64 consecutive u32 words of a
-// residual row (256 bytes, one coalesced wave-wide load).  Each wave keeps eight row loads in flight
-// because the host link's latency, not ALU work, bounds the fetch.  The code is kept small on purpose
+// residual row (256 bytes, one coalesced wave-wide load).  Each wave requests two, four or eight rows per round
+// (the launch's choice): the host link's latency, not ALU work, bounds the fetch, and the link serves only so many
+// bytes per round trip.  The code is kept small on purpose
 // (rolled loops, one code path): a DEC workgroup runs its instructions once, so every instruction
 // cache line it touches is a cold miss on the critical path.
 //
@@ -39,6 +40,7 @@ struct DecParams {
     uint32_t segs_per_block;    // ceil(nseg / sg)
     uint32_t slots_per_block;   // capacity of the per-workgroup row list
     uint32_t fused_select;      // 1: select in-kernel; 0: row indices supplied in sel_rows
+    uint32_t rows_in_flight;    // residual rows a wave requests at a time: 2, 4 or 8 (dec_fetch_rows)
     unsigned long long* trace;  // optional [workgroup][8] cycle stamps of the phases (diagnostics), or null
 };
 
@@ -514,11 +516,47 @@ __device__ __forceinline__ void dec_accumulate_word(uint32_t w, float act, float
     acc[7] += (float)(hi >> 24) * act;
 }
 
+// The rows rl, rl + RL, ... of the workgroup's list for one wave's column of the residual, U requests at a time.  U is
+// the launch's choice (DecParams::rows_in_flight): the host link serves about 140 KB per round trip, and a launch
+// that asks for several times that makes every request wait longer (Llama-3-8B token at k_chunk 32: 2897 us with eight
+// rows per wave and request round, 2801 with two, 2853 with one; at k_chunk 8, where a wave has few rows, four are best).
+template <int U>
+__device__ __forceinline__ void dec_fetch_rows(const uint32_t* base, uint32_t M, uint32_t rl, uint32_t RL, uint32_t nslots,
+                                               const int32_t* lrows, const float* lacts, float (&acc)[8], float& act_sum) {
+#pragma unroll 1
+    for (uint32_t r = rl; r < nslots; r += RL * U) {
+        uint32_t data[U];
+        float act[U];
+        int32_t row[U];
+        // all list entries first (one LDS round trip), then the requests; entries are the same in
+        // every lane, so they live in scalar registers
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t rr = r + (uint32_t)u * RL;
+            const bool valid = rr < nslots;
+            const uint32_t ri = valid ? rr : 0u;
+            const int32_t rw = lrows[ri];
+            const float a = lacts[ri];
+            row[u] = __builtin_amdgcn_readfirstlane(valid ? rw : -1);
+            act[u] = __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(a)));
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (row[u] >= 0) data[u] = base[(size_t)row[u] * M];
+            else { data[u] = 0x88888888u; act[u] = 0.f; }                    // nibble 8 == value 0
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            act_sum += act[u];
+            dec_accumulate_word(data[u], act[u], acc);
+        }
+    }
+}
+
 template <int DT, int NW>
 __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint32_t sgid, uint32_t nslots,
                                           const int32_t* lrows, const float* lacts, float* red) {
     using E = Elem<DT>;
-    constexpr int U = 8;                                // residual rows in flight per wave
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     constexpr uint32_t nw = NW, nt = NW * kWave;
     const uint32_t seg_lo = sgid * p.segs_per_block;
@@ -550,34 +588,9 @@ __device__ __forceinline__ void dec_fetch(const DecParams& p, uint32_t bid, uint
 
         if (col_ok) {
             const uint32_t* base = p.residual + w0;
-#pragma unroll 1
-            for (uint32_t r = rl; r < nslots; r += RL * U) {
-                uint32_t data[U];
-                float act[U];
-                int32_t row[U];
-                // all list entries first (one LDS round trip), then the requests; entries are the same in
-                // every lane, so they live in scalar registers
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const uint32_t rr = r + (uint32_t)u * RL;
-                    const bool valid = rr < nslots;
-                    const uint32_t ri = valid ? rr : 0u;
-                    const int32_t rw = lrows[ri];
-                    const float a = lacts[ri];
-                    row[u] = __builtin_amdgcn_readfirstlane(valid ? rw : -1);
-                    act[u] = __uint_as_float((uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(a)));
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    if (row[u] >= 0) data[u] = base[(size_t)row[u] * p.M];
-                    else { data[u] = 0x88888888u; act[u] = 0.f; }                    // nibble 8 == value 0
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    act_sum += act[u];
-                    dec_accumulate_word(data[u], act[u], acc);
-                }
-            }
+            if (p.rows_in_flight <= 2u) dec_fetch_rows<2>(base, p.M, rl, RL, nslots, lrows, lacts, acc, act_sum);
+            else if (p.rows_in_flight <= 4u) dec_fetch_rows<4>(base, p.M, rl, RL, nslots, lrows, lacts, acc, act_sum);
+            else dec_fetch_rows<8>(base, p.M, rl, RL, nslots, lrows, lacts, acc, act_sum);
         }
         dec_stamp(p, bid, 2);
         // cross-wave reduction through LDS (plain stores; LDS float atomics are slow), then one

@@ -77,6 +77,8 @@ int decdec_version(void);
  *   "dec_block_waves"       waves of a standalone DEC workgroup: 4, 8 or 16 [default]; the launch plan follows.
  *   "dec_force_cg", "dec_force_sg"   DEC launch plans made from now on use this many chunk groups / segment groups
  *                           where the shape allows; 0 = planned [default].
+ *   "dec_rows_in_flight"    residual rows a DEC wave requests per round: 2, 4 or 8; 0 = chosen per launch from the rows
+ *                           per wave and the time the launch occupies the link [default].
  *   "anyprec_rpw", "anyprec_rg", "lutgemm_ktiles", "sqllm_ktiles"   rows per wave / row groups per workgroup / K ranges
  *                           of the base GEMVs; 0 = automatic [default].  (sqllm_ktiles = 1 and lutgemm_ktiles = 1 give
  *                           every output a single atomic add from the GEMV.)

@@ -43,7 +43,8 @@ def test_version_and_options():
     named = set(re.findall(r'"([a-z0-9_]+)"', block))
     defaults = {"fusion": 1, "host_noncoherent": 0, "anyprec_rpw": 0, "anyprec_tile": 0, "lutgemm_ktiles": 0,
                 "sqllm_ktiles": 0, "attention_two_step": 0, "attention_single_below": 512, "fused_two_per_cu": -1, "fused_small": -1, "anyprec_rg": 0, "dec_block_waves": 16,
-                "dec_max_chunk_groups": 0, "gemv_max_k_ranges": 0, "dec_force_cg": 0, "dec_force_sg": 0, "dec_trace": 0}
+                "dec_max_chunk_groups": 0, "gemv_max_k_ranges": 0, "dec_force_cg": 0, "dec_force_sg": 0, "dec_trace": 0,
+                "dec_rows_in_flight": 0}
     assert named == set(defaults), named ^ set(defaults)
     for name, value in defaults.items():
         assert _lib.get_option(name) == value, name

@@ -465,6 +465,40 @@ def test_dec_in_smaller_workgroups(waves, c_oracle):
         _lib.set_option("dec_block_waves", 16)
 
 
+@pytest.mark.parametrize("rows_per_round", [0, 2, 4, 8])
+def test_residual_fetch_with_every_request_width(rows_per_round, c_oracle):
+    """The fetch loop requests 2, 4 or 8 residual rows per wave and round (chosen per launch; option
+    dec_rows_in_flight fixes it): the same outputs whichever it is, with row counts per wave that are not multiples of
+    the width (k_chunk 3, 20, 33), a short last chunk, DEC alone and fused, 16- and 8-wave workgroups."""
+    from decdec_amd import _lib
+    _lib.set_option("dec_rows_in_flight", rows_per_round)
+    try:
+        for K, N, k_chunk, n_tb in [(4096, 4096, 3, 16), (4096, 1024, 33, 8), (14336, 4096, 20, 24), (2048 + 512, 64, 32, 4),
+                                    (4096, 14336, 32, 32)]:
+            L = make_dec_layer(K, N, seed=K + N + k_chunk + 1)
+            ctx, rows, acts = _ctx(n_tb, K, torch.float16)
+            cfg = ext.create_dec_config(ctx, k_chunk, L["cheat"], L["scales"], L["th"])
+            want_rows, _, filled = O.select_channels(np_of(L["x"]), np_of(L["th"]), k_chunk)
+            dec = c_oracle.dec_apply(np_of(L["x"]), L["cheat"].numpy(), np_of(L["scales"]), want_rows[filled])
+            base = c_oracle.anyprec_gemv(np_of(L["x"]), L["qweight"].numpy(), np_of(L["lut"]), 3)
+            for mode in ("dec", "dec8", "fused"):
+                _lib.set_option("dec_block_waves", 8 if mode == "dec8" else 16)
+                rows.fill_(-7)
+                out = torch.zeros(1, 1, N, dtype=torch.float16, device="cuda")
+                if mode == "fused":
+                    ext.dec_anyprec(cfg, L["x"].cuda(), out, L["qweight"].cuda(), L["lut"].cuda(), 3)
+                else:
+                    ext.dec(cfg, L["x"].cuda(), out)
+                torch.cuda.synchronize()
+                got = rows.cpu().numpy()[: want_rows.shape[0]]
+                assert np.array_equal(got[filled], want_rows[filled]), (K, N, k_chunk, mode)
+                check_output(np_of(out).reshape(-1), dec + (base if mode == "fused" else 0.0), "fp16", (K, N, k_chunk, mode, rows_per_round))
+            ext.destroy_dec_config(cfg)
+    finally:
+        _lib.set_option("dec_rows_in_flight", 0)
+        _lib.set_option("dec_block_waves", 16)
+
+
 @pytest.mark.parametrize("waves", [4, 8, 16])
 def test_selection_with_crowded_windows(waves, c_oracle):
     """Activations far weaker than the calibration set: the cut falls among the crowded low buckets, where a bucket
