@@ -575,8 +575,9 @@ def main():
     ap.add_argument("--n-tb", type=int, default=32, help="workgroups DEC may occupy (the sweep shows 8..64)")
     ap.add_argument("--sweep", action="store_true", help="also sweep k_chunk x n_tb (slower)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--leg", choices=["all", "roofline", "kernels", "helpers", "link", "trace"], default="all",
-                    help="roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
+    ap.add_argument("--leg", choices=["all", "token", "roofline", "kernels", "helpers", "link", "trace"], default="all",
+                    help="token: only the token (batched, one launch per layer, graph branches; with DEC and base-only); "
+                         "roofline: only the roofline kernel's launches and a 256 MiB device copy (short run for counter "
                          "collection); kernels: per-kernel table over the configuration shapes (k_chunk 32, n_tb 32); "
                          "helpers: the decode harness's helper kernels (output head, attention, norm, activation); "
                          "link: zero-copy reads of pinned host memory over workgroup counts and request widths; "
@@ -724,6 +725,10 @@ def main():
         "dec_host_link_bytes_per_token": int(host_bytes * scale),
         "dec_host_link_gbs": round(host_bytes / dec_us / 1e3, 2),
     }
+    if args.leg == "token":          # the token three ways and nothing else (a kernel trace of this maps grid sizes to launches)
+        drop_configs(ctxs, cfgs)
+        print(json.dumps(result))
+        return
     result["roofline_link"] = roofline_link_leg(torch, ext, protos, args.k_chunk, args.n_tb, link_leg(torch))
     drop_configs(ctxs, cfgs)
     # Progress against the two floors of the step: the base path against the HBM peak, the compensated step against the

@@ -353,18 +353,20 @@ double dec_residual_rate(const Config* c) { return c->residual_host ? kHostLinkB
 
 // Residual rows a wave requests per round (dec_role.h, dec_fetch_rows): the fewest of 2, 4, 8 with which the wave's rows
 // take no more rounds than fit into the time the launch's rows occupy the link anyway (a round trip under light load is
-// about 1.5 us).  Few rows per round keep the number of requests in flight near what the link serves per round trip;
+// about 2 us).  Few rows per round keep the number of requests in flight near what the link serves per round trip;
 // measured on the Llama-3-8B token with one value for every launch, k_chunk 4 / 8 / 16 / 32 / 64: 1336 / 1496 / 1882 /
 // 2808 / 4767 us with two, 1367 / 1459 / 1917 / 2912 / 4909 with four, 1400 / 1520 / 1935 / 2903 / 4866 with eight
 // (at k_chunk 8 the down projection has eight rows per wave behind 4 us of link time and wants four per round; with the
-// residual in HBM, k_chunk 64: 1874 / 1677 / 1642).
+// residual in HBM, k_chunk 64: 1874 / 1677 / 1642; Phi-3-medium decode with DEC on gate_up and down at k_chunk 8, where a
+// workgroup has 18 segments for 16 waves: 320.8 / 328.5 / 328.6 tokens/s).
 uint32_t dec_rows_per_round(const DecPlan& plan, uint32_t nw, double launch_link_us) {
     if (g_opt.dec_rows_in_flight > 0) return (uint32_t)g_opt.dec_rows_in_flight;
     const uint32_t sb = std::max(1u, std::min(plan.segs_per_block, nw)), waves_per_segment = std::max(1u, nw / sb);
     const uint32_t rows_per_wave = cdiv(plan.slots, waves_per_segment);
-    const uint32_t rounds = (uint32_t)std::max(1.0, launch_link_us / 1.5);
+    const uint32_t passes = cdiv(plan.segs_per_block, nw);            // a workgroup with more segments than waves walks its rows again
+    const uint32_t rounds = (uint32_t)std::max(1.0, launch_link_us / 2.0);
     uint32_t u = 2;
-    while (u < 8u && cdiv(rows_per_wave, u) > rounds) u *= 2u;
+    while (u < 8u && passes * cdiv(rows_per_wave, u) > rounds) u *= 2u;
     return u;
 }
 
