@@ -992,8 +992,17 @@ bool fused_two_per_cu_at(double dec_us, GemvKind kind, double weight_bytes) {
     const double flip = kind == kAnyprec ? 0.9 : (kind == kSqllm ? 1.15 : 1.3);
     return dec_us < flip * gemv_estimate_us(kind, weight_bytes);
 }
+// Rate at which the launch-form rules price a layer's residual rows.  A device-resident residual makes the DEC role the
+// short one for any-precision and LUT-GEMM launches at any k_chunk up to 32 (measured in the decode harness, residual
+// in HBM: Phi-3 LUT-GEMM 284 tokens/s with the two-per-CU instance against 274 without); beside the SqueezeLLM GEMV its
+// role still outlasts the GEMV at k_chunk 32 (8.5 us at 4096 -> 4096, 15.7 us at 14336 -> 4096: about 120 GB/s on top of
+// the floor; Llama-3-8B SqueezeLLM, k_chunk 32 / 8: 468 / 479 tokens/s without the instance, 441 / 521 with it).
+double dec_form_rate(const Config* c, GemvKind kind) {
+    if (c->residual_host) return kHostLinkBytesPerUs;
+    return kind == kSqllm ? 120e3 : kDeviceResidualBytesPerUs;
+}
 bool fused_two_per_cu(const Config* c, GemvKind kind, double weight_bytes) {
-    return fused_two_per_cu_at(dec_estimate_us(c), kind, weight_bytes);
+    return fused_two_per_cu_at(dec_estimate_shape_us(c->K, c->N, c->k_chunk, dec_form_rate(c, kind)), kind, weight_bytes);
 }
 
 // Whether a fused 3-bit any-precision launch runs both roles in workgroups of `nw` waves (the GEMV's standalone
@@ -1289,7 +1298,7 @@ int batch_common(uint32_t n, const uint64_t* configs, const void* input, void* c
         if (have_dec) {
             dec_total += dplan.cg * dplan.sg;
             d.lds = std::max(d.lds, dplan.lds);
-            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_residual_rate(c);
+            dec_us += (double)((uint64_t)c->k_chunk * c->K / 1024u) * (double)c->N * 0.5 / dec_form_rate(c, kind);
             any_dec = true;
         }
         gemv_total += ld.grid;
